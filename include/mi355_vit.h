@@ -1,0 +1,183 @@
+/*
+ * libmi355vit -- C ABI of the MI355X (gfx950) kernels behind the Qwen2.5-VL
+ * vision-tower forward/backward.
+ *
+ * The reference (ray-project/multimodal-training) has no native boundary on
+ * this path: every entry point below replaces a span of PyTorch/ATen calls in
+ * the reference's Python, cited as file:line relative to the reference root
+ * ("modeling" = python/models/qwen2_5_vl/modeling_qwen2_5_vl.py, "spu" =
+ * python/models/qwen2_5_vl/sequence_parallel_utils.py, "[tf]" = transformers
+ * models/qwen2/modeling_qwen2.py).
+ *
+ * Conventions
+ *   - every function returns 0 on success or a negative MVIT_ERR_* code;
+ *     mvit_last_error() then holds a message (thread-local);
+ *   - nothing here allocates, frees or synchronises: the caller passes every
+ *     output and workspace buffer and the HIP stream to enqueue on;
+ *   - all pointers are device pointers unless the parameter says "host";
+ *   - `dtype` is MVIT_F32 or MVIT_BF16 (storage type of activations/weights;
+ *     accumulation is always fp32);
+ *   - row-major everywhere; `ld*` / `*_stride` are in elements.
+ */
+#ifndef MI355_VIT_H
+#define MI355_VIT_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* mvit_stream_t; /* hipStream_t */
+
+enum { MVIT_F32 = 0, MVIT_BF16 = 1 };
+enum { MVIT_OK = 0, MVIT_ERR_ARG = -1, MVIT_ERR_LAUNCH = -2, MVIT_ERR_UNSUPPORTED = -3 };
+
+int mvit_version(void);
+const char* mvit_last_error(void);
+
+/* ---------------------------------------------------------------- host planners (integer, bit-exact) */
+
+/* Position ids (h, w) of every patch in 2x2-merge-block order, repeated per frame.
+ * Replaces rot_pos_emb's index construction, modeling:841-864.
+ * grid_thw: host [n,3] int64; pos_ids: host [S,2] int64 with S = sum t*h*w. */
+int mvit_rot_pos_ids(const int64_t* grid_thw, int64_t n, int merge, int64_t* pos_ids);
+
+/* Window permutation of merged units and cumulative window lengths in patches with
+ * consecutive duplicates removed.  Replaces get_window_index + unique_consecutive,
+ * modeling:870-909 and :927-932.
+ * window_index: host [S/merge^2] int64; cu_window: host int32 buffer of capacity cu_cap
+ * (S/merge^2 + 1 always suffices); *n_cu receives the entry count. */
+int mvit_window_index(const int64_t* grid_thw, int64_t n, int merge, int window_size, int patch_size,
+                      int64_t* window_index, int32_t* cu_window, int64_t cu_cap, int64_t* n_cu);
+
+/* cu_seqlens = [0, cumsum(repeat_interleave(h*w, t))], modeling:944-952.  cu: host int32 [sum t + 1]. */
+int mvit_cu_seqlens(const int64_t* grid_thw, int64_t n, int32_t* cu, int64_t cu_cap, int64_t* n_cu);
+
+/* Token-granular cut positions, spu:105-114.  cuts: host int64 [sp+1]. */
+int mvit_sp_token_cuts(int64_t sample_len, int sp, int64_t* cuts);
+
+/* Window-aligned cut positions, spu:117-164.  cut_pos, cut_idx: host int64 [sp+1]. */
+int mvit_sp_window_cuts(int64_t sample_len, int sp, const int64_t* window_lengths, int64_t n_windows,
+                        int64_t* cut_pos, int64_t* cut_idx);
+
+/* ---------------------------------------------------------------- bandwidth-bound kernels */
+
+/* y = w * cast(x_f32 * rsqrt(mean(x_f32^2) + eps)); rstd[rows] (fp32) is saved for the backward.
+ * Replaces Qwen2RMSNorm.forward, [tf]:247-252 (call sites modeling:771-772, :253). */
+int mvit_rmsnorm_fwd(const void* x, const void* w, void* y, float* rstd, int64_t rows, int64_t cols,
+                     float eps, int dtype, mvit_stream_t stream);
+
+/* dx = [dx_add +] rstd * (dy*w - xhat * mean(dy*w*xhat)),  dw_partial[b, :] = sum over block b's rows of dy*xhat.
+ * The autograd backward of the same lines.  dx_add may be null; dx may alias dx_add.
+ * dw_partial: fp32 [n_partial, cols]; reduce it with mvit_reduce_partials. */
+int mvit_rmsnorm_bwd(const void* dy, const void* x, const void* w, const float* rstd, const void* dx_add,
+                     void* dx, float* dw_partial, int n_partial, int64_t rows, int64_t cols, int dtype,
+                     mvit_stream_t stream);
+
+/* out[c] = sum_b partial[b, c], written as `out_dtype`. */
+int mvit_reduce_partials(const float* partial, int n_partial, int64_t cols, void* out, int out_dtype,
+                         mvit_stream_t stream);
+
+/* In-place rotary embedding of `nheads` heads of `head_dim` laid out at x[row*row_stride + h*head_dim + j]:
+ *   out[j]        = x[j]*cos[j]               - x[j+half]*sin[j]
+ *   out[j+half]   = x[j+half]*cos[j+half]     + x[j]*sin[j+half]
+ * backward != 0 applies the transposed map (the gradient).  cos, sin: fp32 [rows, head_dim].
+ * Replaces apply_rotary_pos_emb_vision / rotate_half, modeling:265-283. */
+int mvit_rope(void* x, const float* cos, const float* sin, int64_t rows, int nheads, int head_dim,
+              int64_t row_stride, int backward, int dtype, mvit_stream_t stream);
+
+/* dst[i, :] = src[index[i], :] for rows of row_bytes bytes (multiple of 4).  Bit-exact.
+ * Replaces the window reorder x.view(M,4,C)[window_index] and its inverse, modeling:934-940, :1067-1068. */
+int mvit_gather_rows(const void* src, const int64_t* index, void* dst, int64_t n_rows, int64_t row_bytes,
+                     mvit_stream_t stream);
+
+/* For each of nseg descriptors (src_row, dst_row, n_rows) (device int64 [nseg,3]) copy n_rows rows of
+ * row_bytes bytes.  Bit-exact.  Replaces the torch.cat of slices in split_pack_by_sp (spu:265-269),
+ * unpad_batch_to_pack (spu:342-346), build_local_rope (spu:395-404) and the re-interleave after the
+ * ragged all-gather (modeling:1040-1064).  max_seg_rows bounds n_rows (grid sizing). */
+int mvit_segment_copy(const void* src, void* dst, const int64_t* desc, int64_t nseg, int64_t max_seg_rows,
+                      int64_t row_bytes, mvit_stream_t stream);
+
+/* pack [sum len, row] -> padded [B, pad_len, row] filled with `pad_value` past each sample's length,
+ * plus mask [B, pad_len] (uint8 0/1).  lens, offsets: device int64 [B].  elem_size 2 or 4; pad_bits is
+ * the bit pattern of the pad value in that element type.  Replaces pad_pack_to_batch, spu:300-327. */
+int mvit_pad_pack(const void* pack, void* padded, uint8_t* mask, const int64_t* lens, const int64_t* offsets,
+                  int64_t batch, int64_t pad_len, int64_t row_elems, int elem_size, uint32_t pad_bits,
+                  mvit_stream_t stream);
+
+/* dst = cast(src) element-wise between MVIT_F32 and MVIT_BF16 over a [rows, cols] view with row strides. */
+int mvit_cast2d(const void* src, int64_t src_ld, int src_dtype, void* dst, int64_t dst_ld, int dst_dtype,
+                int64_t rows, int64_t cols, mvit_stream_t stream);
+
+/* out[c] (+)= sum_r x[r, c]; fp32 partials [n_partial, cols], reduce with mvit_reduce_partials.
+ * Bias gradients of the Linear layers (autograd of modeling:395-397, :471, :204, :255-257). */
+int mvit_colsum(const void* x, int64_t ld, int64_t rows, int64_t cols, float* partial, int n_partial, int dtype,
+                mvit_stream_t stream);
+
+/* ---------------------------------------------------------------- MFMA GEMM with fused epilogues */
+
+enum {
+  MVIT_EPI_NONE = 0,       /* C = acc                                                         */
+  MVIT_EPI_BIAS = 1,       /* C = acc + bias[n]                                               */
+  MVIT_EPI_BIAS_RES = 2,   /* C = acc + bias[n] + R[m,n]                                      */
+  MVIT_EPI_BIAS_GELU = 3,  /* aux = acc + bias[n];  C = gelu_erf(aux)                         */
+  MVIT_EPI_SWIGLU = 4,     /* g = acc(B)+bias, u = acc(B2)+bias2; aux[m,n]=g, aux[m,aux_off+n]=u; C = silu(g)*u */
+  MVIT_EPI_SWIGLU_BWD = 5, /* dh = acc; (g,u) = R[m,n], R[m,aux_off+n]; C[m,n]=dg, C[m,aux_off+n]=du */
+  MVIT_EPI_GELU_BWD = 6,   /* C = acc * gelu_erf'(R[m,n])                                     */
+  MVIT_EPI_ACCUM = 7       /* C = C + acc                                                     */
+};
+
+typedef struct mvit_gemm_args {
+  int dtype;     /* of A, B, B2, R, aux */
+  int out_dtype; /* of C */
+  int trans_a;   /* 0: A is [M,K] (lda >= K);  1: A is [K,M] (lda >= M) */
+  int trans_b;   /* 0: B is [N,K] (ldb >= K);  1: B is [K,N] (ldb >= N) */
+  int epilogue;  /* MVIT_EPI_* */
+  int reserved;
+  int64_t M, N, K;
+  const void* A;
+  int64_t lda;
+  const void* B;
+  const void* B2; /* SWIGLU only; same ldb */
+  int64_t ldb;
+  const void* bias;  /* [N], dtype; may be null for NONE/ACCUM/..._BWD */
+  const void* bias2; /* SWIGLU only */
+  void* C;
+  int64_t ldc;
+  const void* R; /* residual / saved pre-activation */
+  int64_t ldr;
+  void* aux;
+  int64_t ldaux;
+  int64_t aux_off; /* column offset of the second half in aux (SWIGLU) / R and C (SWIGLU_BWD) */
+} mvit_gemm_args;
+
+/* C[M,N] = epilogue(sum_k A[m,k] * B[n,k]).  Operands must be 16-byte aligned with lda/ldb multiples of
+ * 16 bytes; K need not be a multiple of the tile (zero-filled).  Replaces nn.Linear / Conv3d(k==s) and
+ * their autograd: modeling:230 (patch embed), :395-397 (q/k/v), :471 (proj), :204 (SwiGLU MLP), :261
+ * (merger), with the element-wise ops of :204, :256, :784, :791 fused as epilogues. */
+int mvit_gemm(const mvit_gemm_args* args, mvit_stream_t stream);
+
+/* ---------------------------------------------------------------- varlen attention */
+
+/* Per segment [cu[i], cu[i+1]) and head: O = softmax(Q K^T * scale) V, non-causal, fp32 softmax;
+ * lse[h, s] = log sum exp of the scaled scores (fp32 [nheads, total]).
+ * q/k/v/o element (s, h, j) lives at ptr[s*row_stride + h*head_dim + j].
+ * Replaces the attention-backend call of _forward_standard, modeling:427-468 (eager: :298-321), and of
+ * the sequence-parallel full-attention core, modeling:664-731 (nheads = heads / sp). */
+int mvit_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* cu_seqlens,
+                  int n_seg, int max_seqlen, int64_t total, int nheads, int head_dim, int64_t q_stride,
+                  int64_t k_stride, int64_t v_stride, int64_t o_stride, float scale, int dtype,
+                  mvit_stream_t stream);
+
+/* Gradients of the above.  delta: fp32 workspace [nheads, total].  dq/dk/dv use the q/k/v strides given. */
+int mvit_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                  void* dq, void* dk, void* dv, float* delta, const int32_t* cu_seqlens, int n_seg,
+                  int max_seqlen, int64_t total, int nheads, int head_dim, int64_t q_stride, int64_t k_stride,
+                  int64_t v_stride, int64_t o_stride, int64_t do_stride, int64_t dq_stride, int64_t dk_stride,
+                  int64_t dv_stride, float scale, int dtype, mvit_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_VIT_H */

@@ -1,0 +1,779 @@
+// Variable-length (cu_seqlens) non-causal attention, forward and backward, for gfx950.
+//
+// bf16 path: flash-style kernels on v_mfma_f32_16x16x32_bf16 (+ one 16x16x16 step when head_dim/16 is odd,
+// so head_dim 80 = 5 x 16 is contracted exactly, no padding).  All products are oriented so that the
+// accumulator layout of one MFMA is directly the B-operand layout of the next:
+//   forward : S^T = K Q^T   (lane: query l%16, keys 4*(l/16)+i)  ->  O^T += V^T P^T
+//   dK/dV   : S = Q K^T, dP = dO V^T (lane: key l%16, queries 4*(l/16)+i)  ->  dV^T += dO^T P, dK^T += Q^T dS
+//   dQ      : S^T, dP^T as in the forward  ->  dQ^T += K^T dS^T
+// Operands that are needed "transposed" (V, dO, Q, K as the left factor of the second product) are read
+// from their natural [row][head_dim] LDS tiles with ds_read_b64_tr_b16.  Softmax statistics live in
+// registers; row reductions are two cross-lane exchanges (lanes l, l^16, l^32, l^48 share a query).
+// The backward is split in two kernels (dK/dV, then dQ), which keeps it free of atomics and bit-reproducible.
+//
+// fp32 path (parity mode): one lane per query (or key) row, K/V (or Q/dO) tiles broadcast from LDS.
+#include "mvit_common.h"
+
+namespace {
+
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+
+struct AttnParams {
+  const void *q, *k, *v, *o, *d_o;
+  void *out, *dq, *dk, *dv;
+  float* lse;
+  float* delta;
+  const int32_t* cu;
+  int64_t total;
+  int nheads;
+  int64_t q_stride, k_stride, v_stride, o_stride, do_stride, dq_stride, dk_stride, dv_stride;
+  float scale;
+};
+
+typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ bf16x8 tr_pair(const bf16_t* p0, const bf16_t* p1) {
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)p0);
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)p1);
+  s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(bf16x8, both);
+}
+__device__ __forceinline__ bf16x8 pack8(const f32x4& a, const f32x4& b) {
+  bf16x8 r;
+  r[0] = (bf16_t)a[0]; r[1] = (bf16_t)a[1]; r[2] = (bf16_t)a[2]; r[3] = (bf16_t)a[3];
+  r[4] = (bf16_t)b[0]; r[5] = (bf16_t)b[1]; r[6] = (bf16_t)b[2]; r[7] = (bf16_t)b[3];
+  return r;
+}
+__device__ __forceinline__ f32x4 mfma32(const bf16x8& a, const bf16x8& b, const f32x4& c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mfma16(const bf16x4& a, const bf16x4& b, const f32x4& c) {
+  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+}
+
+template <int ND>
+struct Geo {
+  static constexpr int HD = 16 * ND;
+  static constexpr int NK32 = ND / 2;         // 32-wide contraction steps over head_dim
+  static constexpr bool TAIL16 = (ND & 1);    // plus one 16-wide step
+  static constexpr int PK = HD + 8;           // pitch of tiles read with 16-byte row loads
+  static constexpr int PV = (HD % 32 == 0) ? HD + 16 : HD;  // pitch of tiles read only through transposing loads
+  static constexpr int CH = 2 * ND;           // 16-byte chunks per row
+};
+
+// Operand fragments of 16 rows x head_dim for one lane, in the "row l%16, contraction 8*(l/16)+j" layout
+// (serves as MFMA A for rows, or as MFMA B for columns).
+template <int ND>
+struct RowFrag {
+  bf16x8 k32[Geo<ND>::NK32 > 0 ? Geo<ND>::NK32 : 1];
+  bf16x4 k16;
+};
+
+template <int ND>
+__device__ __forceinline__ void load_rowfrag_global(RowFrag<ND>& f, const bf16_t* row_ptr, bool valid, int g) {
+  using G = Geo<ND>;
+#pragma unroll
+  for (int ks = 0; ks < G::NK32; ++ks) {
+    bf16x8 v;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (bf16_t)0.f;
+    if (valid) v = *reinterpret_cast<const bf16x8*>(row_ptr + 32 * ks + 8 * g);
+    f.k32[ks] = v;
+  }
+  if (G::TAIL16) {
+    bf16x4 v = {(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
+    if (valid) v = *reinterpret_cast<const bf16x4*>(row_ptr + 32 * G::NK32 + 4 * g);
+    f.k16 = v;
+  }
+}
+template <int ND, int PITCH>
+__device__ __forceinline__ void load_rowfrag_lds(RowFrag<ND>& f, const bf16_t* tile, int row, int g) {
+  using G = Geo<ND>;
+  const bf16_t* p = tile + row * PITCH;
+#pragma unroll
+  for (int ks = 0; ks < G::NK32; ++ks) f.k32[ks] = *reinterpret_cast<const bf16x8*>(p + 32 * ks + 8 * g);
+  if (G::TAIL16) f.k16 = *reinterpret_cast<const bf16x4*>(p + 32 * G::NK32 + 4 * g);
+}
+// acc += rows(a) . rows(b)^T over head_dim  (16x16 tile)
+template <int ND>
+__device__ __forceinline__ f32x4 dot_frag(const RowFrag<ND>& a, const RowFrag<ND>& b) {
+  using G = Geo<ND>;
+  f32x4 c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int ks = 0; ks < G::NK32; ++ks) c = mfma32(a.k32[ks], b.k32[ks], c);
+  if (G::TAIL16) c = mfma16(a.k16, b.k16, c);
+  return c;
+}
+
+// Cooperative global -> LDS copy of `rows` x head_dim (zero-filled past `valid_rows`).
+template <int ND, int PITCH, int NTHREADS>
+__device__ __forceinline__ void stage_tile(bf16_t* tile, const bf16_t* src, int64_t stride, int rows, int valid_rows) {
+  using G = Geo<ND>;
+  const int nchunks = rows * G::CH;
+  for (int c = threadIdx.x; c < nchunks; c += NTHREADS) {
+    const int r = c / G::CH, dc = c % G::CH;
+    bf16x8 v;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (bf16_t)0.f;
+    if (r < valid_rows) v = *reinterpret_cast<const bf16x8*>(src + (int64_t)r * stride + dc * 8);
+    *reinterpret_cast<bf16x8*>(tile + r * PITCH + dc * 8) = v;
+  }
+}
+
+// ================================================================================================
+// Forward.  Block = NWAVES waves = 64*NWAVES queries of one (segment, head); 64 keys per iteration.
+template <int ND, int NWAVES>
+__global__ __launch_bounds__(64 * NWAVES) void attn_fwd_mfma(const AttnParams p) {
+  using G = Geo<ND>;
+  constexpr int HD = G::HD, BNK = 64, NT = 64 * NWAVES;
+  __shared__ __attribute__((aligned(16))) bf16_t lds_k[BNK * G::PK];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_v[BNK * G::PV];
+
+  const int seg = blockIdx.y, h = blockIdx.z;
+  const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
+  const int blk_q0 = blockIdx.x * NT;
+  if (blk_q0 >= L) return;
+  const int l = threadIdx.x & 63, wv = threadIdx.x >> 6, g = l >> 4, r = l & 15;
+  const int q0 = blk_q0 + wv * 64;
+
+  const bf16_t* Q = static_cast<const bf16_t*>(p.q) + (int64_t)s0 * p.q_stride + (int64_t)h * HD;
+  const bf16_t* K = static_cast<const bf16_t*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD;
+  const bf16_t* V = static_cast<const bf16_t*>(p.v) + (int64_t)s0 * p.v_stride + (int64_t)h * HD;
+
+  RowFrag<ND> qf[4];
+#pragma unroll
+  for (int qb = 0; qb < 4; ++qb) {
+    const int qi = q0 + qb * 16 + r;
+    load_rowfrag_global<ND>(qf[qb], Q + (int64_t)qi * p.q_stride, qi < L, g);
+  }
+
+  f32x4 o[4][ND];
+  float m_run[4], l_run[4];
+#pragma unroll
+  for (int qb = 0; qb < 4; ++qb) {
+    m_run[qb] = -INFINITY;
+    l_run[qb] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt) o[qb][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const float c = p.scale * LOG2E;
+
+  for (int k0 = 0; k0 < L; k0 += BNK) {
+    __syncthreads();
+    const int valid = min(BNK, L - k0);
+    stage_tile<ND, G::PK, NT>(lds_k, K + (int64_t)k0 * p.k_stride, p.k_stride, BNK, valid);
+    stage_tile<ND, G::PV, NT>(lds_v, V + (int64_t)k0 * p.v_stride, p.v_stride, BNK, valid);
+    __syncthreads();
+
+    // scores: s[qb][kt][i] = S[query qb*16 + r][key kt*16 + 4g + i]
+    f32x4 s[4][4];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+      RowFrag<ND> kf;
+      load_rowfrag_lds<ND, G::PK>(kf, lds_k, kt * 16 + r, g);
+#pragma unroll
+      for (int qb = 0; qb < 4; ++qb) s[qb][kt] = dot_frag<ND>(kf, qf[qb]);
+    }
+    bf16x8 pb[4][2];
+#pragma unroll
+    for (int qb = 0; qb < 4; ++qb) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const bool ok = (kt * 16 + 4 * g + i) < valid;
+          s[qb][kt][i] = ok ? s[qb][kt][i] * c : -INFINITY;
+          mx = fmaxf(mx, s[qb][kt][i]);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run[qb], mx);  // finite: every tile holds at least one valid key
+      const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_new);
+      m_run[qb] = m_new;
+      float ps = 0.f;
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float e = __builtin_amdgcn_exp2f(s[qb][kt][i] - m_new);
+          s[qb][kt][i] = e;
+          ps += e;
+        }
+      l_run[qb] = l_run[qb] * alpha + ps;
+#pragma unroll
+      for (int dt = 0; dt < ND; ++dt) o[qb][dt] *= alpha;
+      pb[qb][0] = pack8(s[qb][0], s[qb][1]);
+      pb[qb][1] = pack8(s[qb][2], s[qb][3]);
+    }
+    // O^T[d][q] += sum_key V[key][d] P[q][key]; contraction slots (g, j): keys t0*16+4g+j | t1*16+4g+j-4
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int dt = 0; dt < ND; ++dt) {
+        const bf16_t* a0 = lds_v + ((2 * kk) * 16 + 4 * g + (r >> 2)) * G::PV + 16 * dt + 4 * (r & 3);
+        const bf16x8 vf = tr_pair(a0, a0 + 16 * G::PV);
+#pragma unroll
+        for (int qb = 0; qb < 4; ++qb) o[qb][dt] = mfma32(vf, pb[qb][kk], o[qb][dt]);
+      }
+  }
+
+  bf16_t* O = static_cast<bf16_t*>(p.out) + (int64_t)s0 * p.o_stride + (int64_t)h * HD;
+#pragma unroll
+  for (int qb = 0; qb < 4; ++qb) {
+    float lt = l_run[qb];
+    lt += __shfl_xor(lt, 16, 64);
+    lt += __shfl_xor(lt, 32, 64);
+    const int qi = q0 + qb * 16 + r;
+    if (qi < L) {
+      const float inv = 1.f / lt;
+#pragma unroll
+      for (int dt = 0; dt < ND; ++dt) {
+        bf16x4 ov;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ov[i] = (bf16_t)(o[qb][dt][i] * inv);
+        *reinterpret_cast<bf16x4*>(O + (int64_t)qi * p.o_stride + 16 * dt + 4 * g) = ov;
+      }
+      if (g == 0) p.lse[(int64_t)h * p.total + s0 + qi] = (m_run[qb] + __builtin_amdgcn_logf(lt)) * LN2;
+    }
+  }
+}
+
+// delta[h, s] = sum_d O[s,h,d] * dO[s,h,d]
+template <typename T>
+__global__ __launch_bounds__(256) void attn_delta_kernel(const T* __restrict__ o, const T* __restrict__ d_o,
+                                                         float* __restrict__ delta, int64_t total, int nheads, int hd,
+                                                         int64_t o_stride, int64_t do_stride) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total * nheads) return;
+  const int64_t s = i / nheads;
+  const int h = (int)(i % nheads);
+  const T* a = o + s * o_stride + (int64_t)h * hd;
+  const T* b = d_o + s * do_stride + (int64_t)h * hd;
+  float acc = 0.f;
+  for (int j = 0; j < hd; ++j) acc += to_f32(a[j]) * to_f32(b[j]);
+  delta[(int64_t)h * total + s] = acc;
+}
+
+// ================================================================================================
+// dK, dV.  Block = 64*NWAVES keys of one (segment, head); 32 queries per iteration.
+template <int ND, int NWAVES>
+__global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnParams p) {
+  using G = Geo<ND>;
+  constexpr int HD = G::HD, BQ = 32, NT = 64 * NWAVES;
+  __shared__ __attribute__((aligned(16))) bf16_t lds_q[BQ * G::PK];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_do[BQ * G::PK];
+  __shared__ __attribute__((aligned(16))) float lds_lse[BQ];
+  __shared__ __attribute__((aligned(16))) float lds_delta[BQ];
+
+  const int seg = blockIdx.y, h = blockIdx.z;
+  const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
+  const int blk_k0 = blockIdx.x * NT;
+  if (blk_k0 >= L) return;
+  const int l = threadIdx.x & 63, wv = threadIdx.x >> 6, g = l >> 4, r = l & 15;
+  const int key0 = blk_k0 + wv * 64;
+
+  const bf16_t* Q = static_cast<const bf16_t*>(p.q) + (int64_t)s0 * p.q_stride + (int64_t)h * HD;
+  const bf16_t* K = static_cast<const bf16_t*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD;
+  const bf16_t* V = static_cast<const bf16_t*>(p.v) + (int64_t)s0 * p.v_stride + (int64_t)h * HD;
+  const bf16_t* DO = static_cast<const bf16_t*>(p.d_o) + (int64_t)s0 * p.do_stride + (int64_t)h * HD;
+  const float* LSE = p.lse + (int64_t)h * p.total + s0;
+  const float* DELTA = p.delta + (int64_t)h * p.total + s0;
+
+  RowFrag<ND> kf[4], vf[4];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) {
+    const int ki = key0 + kb * 16 + r;
+    load_rowfrag_global<ND>(kf[kb], K + (int64_t)ki * p.k_stride, ki < L, g);
+    load_rowfrag_global<ND>(vf[kb], V + (int64_t)ki * p.v_stride, ki < L, g);
+  }
+  f32x4 dk[4][ND], dv[4][ND];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt) {
+      dk[kb][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      dv[kb][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  const float c = p.scale * LOG2E;
+
+  for (int qs = 0; qs < L; qs += BQ) {
+    __syncthreads();
+    const int valid = min(BQ, L - qs);
+    stage_tile<ND, G::PK, NT>(lds_q, Q + (int64_t)qs * p.q_stride, p.q_stride, BQ, valid);
+    stage_tile<ND, G::PK, NT>(lds_do, DO + (int64_t)qs * p.do_stride, p.do_stride, BQ, valid);
+    if (threadIdx.x < BQ) {
+      const bool ok = (int)threadIdx.x < valid;
+      lds_lse[threadIdx.x] = ok ? LSE[qs + threadIdx.x] * LOG2E : INFINITY;  // +inf => p = 0 for padded queries
+      lds_delta[threadIdx.x] = ok ? DELTA[qs + threadIdx.x] : 0.f;
+    }
+    __syncthreads();
+
+    RowFrag<ND> qa[2], da[2];  // natural-layout A operands: row = query t*16 + r
+    bf16x8 qt[ND], dt_[ND];    // transposed A operands: row = head-dim 16*dt + r, slots = queries
+    f32x4 lse2[2], dl[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      load_rowfrag_lds<ND, G::PK>(qa[t], lds_q, t * 16 + r, g);
+      load_rowfrag_lds<ND, G::PK>(da[t], lds_do, t * 16 + r, g);
+      lse2[t] = *reinterpret_cast<const f32x4*>(lds_lse + t * 16 + 4 * g);
+      dl[t] = *reinterpret_cast<const f32x4*>(lds_delta + t * 16 + 4 * g);
+    }
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {
+      const int off = (4 * g + (r >> 2)) * G::PK + 16 * d + 4 * (r & 3);
+      qt[d] = tr_pair(lds_q + off, lds_q + off + 16 * G::PK);
+      dt_[d] = tr_pair(lds_do + off, lds_do + off + 16 * G::PK);
+    }
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      f32x4 pv[2], ds[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const f32x4 s = dot_frag<ND>(qa[t], kf[kb]);   // S[q = t*16+4g+i][key = kb*16+r]
+        const f32x4 dp = dot_frag<ND>(da[t], vf[kb]);  // dP, same layout
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float e = __builtin_amdgcn_exp2f(s[i] * c - lse2[t][i]);
+          pv[t][i] = e;
+          ds[t][i] = e * (dp[i] - dl[t][i]);
+        }
+      }
+      const bf16x8 pb = pack8(pv[0], pv[1]);
+      const bf16x8 dsb = pack8(ds[0], ds[1]);
+#pragma unroll
+      for (int d = 0; d < ND; ++d) {
+        dv[kb][d] = mfma32(dt_[d], pb, dv[kb][d]);
+        dk[kb][d] = mfma32(qt[d], dsb, dk[kb][d]);
+      }
+    }
+  }
+
+  bf16_t* DK = static_cast<bf16_t*>(p.dk) + (int64_t)s0 * p.dk_stride + (int64_t)h * HD;
+  bf16_t* DV = static_cast<bf16_t*>(p.dv) + (int64_t)s0 * p.dv_stride + (int64_t)h * HD;
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) {
+    const int ki = key0 + kb * 16 + r;
+    if (ki < L) {
+#pragma unroll
+      for (int d = 0; d < ND; ++d) {
+        bf16x4 a, b;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          a[i] = (bf16_t)(dk[kb][d][i] * p.scale);
+          b[i] = (bf16_t)dv[kb][d][i];
+        }
+        *reinterpret_cast<bf16x4*>(DK + (int64_t)ki * p.dk_stride + 16 * d + 4 * g) = a;
+        *reinterpret_cast<bf16x4*>(DV + (int64_t)ki * p.dv_stride + 16 * d + 4 * g) = b;
+      }
+    }
+  }
+}
+
+// ================================================================================================
+// dQ.  Block = 64*NWAVES queries of one (segment, head); 32 keys per iteration.
+template <int ND, int NWAVES>
+__global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams p) {
+  using G = Geo<ND>;
+  constexpr int HD = G::HD, BK = 32, NT = 64 * NWAVES;
+  __shared__ __attribute__((aligned(16))) bf16_t lds_k[BK * G::PK];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_v[BK * G::PK];
+
+  const int seg = blockIdx.y, h = blockIdx.z;
+  const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
+  const int blk_q0 = blockIdx.x * NT;
+  if (blk_q0 >= L) return;
+  const int l = threadIdx.x & 63, wv = threadIdx.x >> 6, g = l >> 4, r = l & 15;
+  const int q0 = blk_q0 + wv * 64;
+
+  const bf16_t* Q = static_cast<const bf16_t*>(p.q) + (int64_t)s0 * p.q_stride + (int64_t)h * HD;
+  const bf16_t* K = static_cast<const bf16_t*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD;
+  const bf16_t* V = static_cast<const bf16_t*>(p.v) + (int64_t)s0 * p.v_stride + (int64_t)h * HD;
+  const bf16_t* DO = static_cast<const bf16_t*>(p.d_o) + (int64_t)s0 * p.do_stride + (int64_t)h * HD;
+  const float* LSE = p.lse + (int64_t)h * p.total + s0;
+  const float* DELTA = p.delta + (int64_t)h * p.total + s0;
+
+  RowFrag<ND> qf[4], dof[4];
+  float lse2[4], dl[4];
+#pragma unroll
+  for (int qb = 0; qb < 4; ++qb) {
+    const int qi = q0 + qb * 16 + r;
+    const bool ok = qi < L;
+    load_rowfrag_global<ND>(qf[qb], Q + (int64_t)qi * p.q_stride, ok, g);
+    load_rowfrag_global<ND>(dof[qb], DO + (int64_t)qi * p.do_stride, ok, g);
+    lse2[qb] = ok ? LSE[qi] * LOG2E : INFINITY;
+    dl[qb] = ok ? DELTA[qi] : 0.f;
+  }
+  f32x4 dq[4][ND];
+#pragma unroll
+  for (int qb = 0; qb < 4; ++qb)
+#pragma unroll
+    for (int d = 0; d < ND; ++d) dq[qb][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const float c = p.scale * LOG2E;
+
+  for (int k0 = 0; k0 < L; k0 += BK) {
+    __syncthreads();
+    const int valid = min(BK, L - k0);
+    stage_tile<ND, G::PK, NT>(lds_k, K + (int64_t)k0 * p.k_stride, p.k_stride, BK, valid);
+    stage_tile<ND, G::PK, NT>(lds_v, V + (int64_t)k0 * p.v_stride, p.v_stride, BK, valid);
+    __syncthreads();
+
+    RowFrag<ND> ka[2], va[2];
+    bf16x8 kt[ND];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      load_rowfrag_lds<ND, G::PK>(ka[t], lds_k, t * 16 + r, g);
+      load_rowfrag_lds<ND, G::PK>(va[t], lds_v, t * 16 + r, g);
+    }
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {
+      const int off = (4 * g + (r >> 2)) * G::PK + 16 * d + 4 * (r & 3);
+      kt[d] = tr_pair(lds_k + off, lds_k + off + 16 * G::PK);
+    }
+#pragma unroll
+    for (int qb = 0; qb < 4; ++qb) {
+      f32x4 ds[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const f32x4 s = dot_frag<ND>(ka[t], qf[qb]);    // S[q = qb*16+r][key = t*16+4g+i]
+        const f32x4 dp = dot_frag<ND>(va[t], dof[qb]);  // dP, same layout
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const bool ok = (t * 16 + 4 * g + i) < valid;
+          const float e = ok ? __builtin_amdgcn_exp2f(s[i] * c - lse2[qb]) : 0.f;
+          ds[t][i] = e * (dp[i] - dl[qb]);
+        }
+      }
+      const bf16x8 dsb = pack8(ds[0], ds[1]);
+#pragma unroll
+      for (int d = 0; d < ND; ++d) dq[qb][d] = mfma32(kt[d], dsb, dq[qb][d]);
+    }
+  }
+
+  bf16_t* DQ = static_cast<bf16_t*>(p.dq) + (int64_t)s0 * p.dq_stride + (int64_t)h * HD;
+#pragma unroll
+  for (int qb = 0; qb < 4; ++qb) {
+    const int qi = q0 + qb * 16 + r;
+    if (qi < L) {
+#pragma unroll
+      for (int d = 0; d < ND; ++d) {
+        bf16x4 a;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[i] = (bf16_t)(dq[qb][d][i] * p.scale);
+        *reinterpret_cast<bf16x4*>(DQ + (int64_t)qi * p.dq_stride + 16 * d + 4 * g) = a;
+      }
+    }
+  }
+}
+
+// ================================================================================================
+// fp32 parity kernels: one lane per row, 32-row tiles of the other side broadcast from LDS.
+template <int HD>
+__global__ __launch_bounds__(64) void attn_fwd_f32(const AttnParams p) {
+  constexpr int TB = 32;
+  __shared__ float sk[TB * HD];
+  __shared__ float sv[TB * HD];
+  const int seg = blockIdx.y, h = blockIdx.z;
+  const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
+  const int q0 = blockIdx.x * 64;
+  if (q0 >= L) return;
+  const int qi = q0 + threadIdx.x;
+  const bool valid = qi < L;
+  const float* Q = static_cast<const float*>(p.q) + (int64_t)s0 * p.q_stride + (int64_t)h * HD;
+  const float* K = static_cast<const float*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD;
+  const float* V = static_cast<const float*>(p.v) + (int64_t)s0 * p.v_stride + (int64_t)h * HD;
+  float qr[HD], acc[HD];
+#pragma unroll
+  for (int j = 0; j < HD; ++j) {
+    qr[j] = valid ? Q[(int64_t)qi * p.q_stride + j] : 0.f;
+    acc[j] = 0.f;
+  }
+  float m = -INFINITY, lsum = 0.f;
+  for (int k0 = 0; k0 < L; k0 += TB) {
+    const int nk = min(TB, L - k0);
+    __syncthreads();
+    for (int i = threadIdx.x; i < TB * HD; i += 64) {
+      const int rr = i / HD, j = i % HD;
+      sk[i] = rr < nk ? K[(int64_t)(k0 + rr) * p.k_stride + j] : 0.f;
+      sv[i] = rr < nk ? V[(int64_t)(k0 + rr) * p.v_stride + j] : 0.f;
+    }
+    __syncthreads();
+    float s[TB];
+    float mx = m;
+#pragma unroll
+    for (int t = 0; t < TB; ++t) {
+      float d = 0.f;
+#pragma unroll
+      for (int j = 0; j < HD; ++j) d += qr[j] * sk[t * HD + j];
+      s[t] = t < nk ? d * p.scale : -INFINITY;
+      mx = fmaxf(mx, s[t]);
+    }
+    const float alpha = expf(m - mx);
+    m = mx;
+    lsum *= alpha;
+#pragma unroll
+    for (int j = 0; j < HD; ++j) acc[j] *= alpha;
+#pragma unroll
+    for (int t = 0; t < TB; ++t) {
+      const float e = expf(s[t] - mx);
+      lsum += e;
+#pragma unroll
+      for (int j = 0; j < HD; ++j) acc[j] += e * sv[t * HD + j];
+    }
+  }
+  if (valid) {
+    float* O = static_cast<float*>(p.out) + (int64_t)(s0 + qi) * p.o_stride + (int64_t)h * HD;
+    const float inv = 1.f / lsum;
+#pragma unroll
+    for (int j = 0; j < HD; ++j) O[j] = acc[j] * inv;
+    p.lse[(int64_t)h * p.total + s0 + qi] = m + logf(lsum);
+  }
+}
+
+template <int HD>
+__global__ __launch_bounds__(64) void attn_bwd_dq_f32(const AttnParams p) {
+  constexpr int TB = 32;
+  __shared__ float sk[TB * HD];
+  __shared__ float sv[TB * HD];
+  const int seg = blockIdx.y, h = blockIdx.z;
+  const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
+  const int q0 = blockIdx.x * 64;
+  if (q0 >= L) return;
+  const int qi = q0 + threadIdx.x;
+  const bool valid = qi < L;
+  const float* Q = static_cast<const float*>(p.q) + (int64_t)s0 * p.q_stride + (int64_t)h * HD;
+  const float* K = static_cast<const float*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD;
+  const float* V = static_cast<const float*>(p.v) + (int64_t)s0 * p.v_stride + (int64_t)h * HD;
+  const float* DO = static_cast<const float*>(p.d_o) + (int64_t)s0 * p.do_stride + (int64_t)h * HD;
+  float qr[HD], dor[HD], acc[HD];
+#pragma unroll
+  for (int j = 0; j < HD; ++j) {
+    qr[j] = valid ? Q[(int64_t)qi * p.q_stride + j] : 0.f;
+    dor[j] = valid ? DO[(int64_t)qi * p.do_stride + j] : 0.f;
+    acc[j] = 0.f;
+  }
+  const float lse = valid ? p.lse[(int64_t)h * p.total + s0 + qi] : INFINITY;
+  const float dl = valid ? p.delta[(int64_t)h * p.total + s0 + qi] : 0.f;
+  for (int k0 = 0; k0 < L; k0 += TB) {
+    const int nk = min(TB, L - k0);
+    __syncthreads();
+    for (int i = threadIdx.x; i < TB * HD; i += 64) {
+      const int rr = i / HD, j = i % HD;
+      sk[i] = rr < nk ? K[(int64_t)(k0 + rr) * p.k_stride + j] : 0.f;
+      sv[i] = rr < nk ? V[(int64_t)(k0 + rr) * p.v_stride + j] : 0.f;
+    }
+    __syncthreads();
+    for (int t = 0; t < nk; ++t) {
+      float d = 0.f, dp = 0.f;
+#pragma unroll
+      for (int j = 0; j < HD; ++j) {
+        d += qr[j] * sk[t * HD + j];
+        dp += dor[j] * sv[t * HD + j];
+      }
+      const float ds = expf(d * p.scale - lse) * (dp - dl);
+#pragma unroll
+      for (int j = 0; j < HD; ++j) acc[j] += ds * sk[t * HD + j];
+    }
+  }
+  if (valid) {
+    float* DQ = static_cast<float*>(p.dq) + (int64_t)(s0 + qi) * p.dq_stride + (int64_t)h * HD;
+#pragma unroll
+    for (int j = 0; j < HD; ++j) DQ[j] = acc[j] * p.scale;
+  }
+}
+
+template <int HD>
+__global__ __launch_bounds__(64) void attn_bwd_dkdv_f32(const AttnParams p) {
+  constexpr int TB = 32;
+  __shared__ float sq[TB * HD];
+  __shared__ float sdo[TB * HD];
+  __shared__ float slse[TB];
+  __shared__ float sdl[TB];
+  const int seg = blockIdx.y, h = blockIdx.z;
+  const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
+  const int kb0 = blockIdx.x * 64;
+  if (kb0 >= L) return;
+  const int ki = kb0 + threadIdx.x;
+  const bool valid = ki < L;
+  const float* Q = static_cast<const float*>(p.q) + (int64_t)s0 * p.q_stride + (int64_t)h * HD;
+  const float* K = static_cast<const float*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD;
+  const float* V = static_cast<const float*>(p.v) + (int64_t)s0 * p.v_stride + (int64_t)h * HD;
+  const float* DO = static_cast<const float*>(p.d_o) + (int64_t)s0 * p.do_stride + (int64_t)h * HD;
+  float kr[HD], vr[HD], dk[HD], dv[HD];
+#pragma unroll
+  for (int j = 0; j < HD; ++j) {
+    kr[j] = valid ? K[(int64_t)ki * p.k_stride + j] : 0.f;
+    vr[j] = valid ? V[(int64_t)ki * p.v_stride + j] : 0.f;
+    dk[j] = 0.f;
+    dv[j] = 0.f;
+  }
+  for (int qs = 0; qs < L; qs += TB) {
+    const int nq = min(TB, L - qs);
+    __syncthreads();
+    for (int i = threadIdx.x; i < TB * HD; i += 64) {
+      const int rr = i / HD, j = i % HD;
+      sq[i] = rr < nq ? Q[(int64_t)(qs + rr) * p.q_stride + j] : 0.f;
+      sdo[i] = rr < nq ? DO[(int64_t)(qs + rr) * p.do_stride + j] : 0.f;
+    }
+    if (threadIdx.x < TB) {
+      const bool ok = (int)threadIdx.x < nq;
+      slse[threadIdx.x] = ok ? p.lse[(int64_t)h * p.total + s0 + qs + threadIdx.x] : INFINITY;
+      sdl[threadIdx.x] = ok ? p.delta[(int64_t)h * p.total + s0 + qs + threadIdx.x] : 0.f;
+    }
+    __syncthreads();
+    for (int t = 0; t < nq; ++t) {
+      float d = 0.f, dp = 0.f;
+#pragma unroll
+      for (int j = 0; j < HD; ++j) {
+        d += sq[t * HD + j] * kr[j];
+        dp += sdo[t * HD + j] * vr[j];
+      }
+      const float e = expf(d * p.scale - slse[t]);
+      const float ds = e * (dp - sdl[t]);
+#pragma unroll
+      for (int j = 0; j < HD; ++j) {
+        dv[j] += e * sdo[t * HD + j];
+        dk[j] += ds * sq[t * HD + j];
+      }
+    }
+  }
+  if (valid) {
+    float* DK = static_cast<float*>(p.dk) + (int64_t)(s0 + ki) * p.dk_stride + (int64_t)h * HD;
+    float* DV = static_cast<float*>(p.dv) + (int64_t)(s0 + ki) * p.dv_stride + (int64_t)h * HD;
+#pragma unroll
+    for (int j = 0; j < HD; ++j) {
+      DK[j] = dk[j] * p.scale;
+      DV[j] = dv[j];
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+inline int pick_waves(int max_seqlen) { return max_seqlen <= 64 ? 1 : (max_seqlen <= 128 ? 2 : 4); }
+
+template <int ND>
+int launch_fwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t s) {
+  const int nw = pick_waves(max_seqlen);
+  dim3 grid((unsigned)((max_seqlen + 64 * nw - 1) / (64 * nw)), (unsigned)n_seg, (unsigned)p.nheads);
+  if (nw == 1) hipLaunchKernelGGL((attn_fwd_mfma<ND, 1>), grid, 64, 0, s, p);
+  else if (nw == 2) hipLaunchKernelGGL((attn_fwd_mfma<ND, 2>), grid, 128, 0, s, p);
+  else hipLaunchKernelGGL((attn_fwd_mfma<ND, 4>), grid, 256, 0, s, p);
+  MVIT_CHECK_LAUNCH("attn_fwd");
+  return MVIT_OK;
+}
+template <int ND>
+int launch_bwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t s) {
+  const int nw = pick_waves(max_seqlen);
+  dim3 grid((unsigned)((max_seqlen + 64 * nw - 1) / (64 * nw)), (unsigned)n_seg, (unsigned)p.nheads);
+  if (nw == 1) {
+    hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 1>), grid, 64, 0, s, p);
+    hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 1>), grid, 64, 0, s, p);
+  } else if (nw == 2) {
+    hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 2>), grid, 128, 0, s, p);
+    hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 2>), grid, 128, 0, s, p);
+  } else {
+    hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 4>), grid, 256, 0, s, p);
+    hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 4>), grid, 256, 0, s, p);
+  }
+  MVIT_CHECK_LAUNCH("attn_bwd");
+  return MVIT_OK;
+}
+template <int HD>
+int launch_f32(const AttnParams& p, int n_seg, int max_seqlen, bool bwd, hipStream_t s) {
+  dim3 grid((unsigned)((max_seqlen + 63) / 64), (unsigned)n_seg, (unsigned)p.nheads);
+  if (!bwd) {
+    hipLaunchKernelGGL((attn_fwd_f32<HD>), grid, 64, 0, s, p);
+  } else {
+    hipLaunchKernelGGL((attn_bwd_dkdv_f32<HD>), grid, 64, 0, s, p);
+    hipLaunchKernelGGL((attn_bwd_dq_f32<HD>), grid, 64, 0, s, p);
+  }
+  MVIT_CHECK_LAUNCH("attn_f32");
+  return MVIT_OK;
+}
+
+int check_common(const char* who, const int32_t* cu, int n_seg, int max_seqlen, int64_t total, int nheads, int head_dim,
+                 int dtype, std::initializer_list<int64_t> strides, std::initializer_list<const void*> ptrs) {
+  MVIT_REQUIRE(cu && n_seg >= 0 && max_seqlen >= 0 && total >= 0 && nheads > 0 && nheads <= 65535 && n_seg <= 65535,
+               "%s: bad sizes (n_seg=%d max_seqlen=%d total=%lld nheads=%d)", who, n_seg, max_seqlen, (long long)total, nheads);
+  MVIT_REQUIRE(dtype == MVIT_BF16 || dtype == MVIT_F32, "%s: dtype %d", who, dtype);
+  MVIT_REQUIRE(head_dim == 32 || head_dim == 64 || head_dim == 80 || head_dim == 128, "%s: head_dim %d not built (32, 64, 80, 128)", who, head_dim);
+  const int vec = dtype == MVIT_BF16 ? 8 : 1;
+  for (int64_t st : strides)
+    MVIT_REQUIRE(st >= (int64_t)nheads * head_dim && st % vec == 0, "%s: row stride %lld must cover %d heads and be a multiple of %d", who, (long long)st, nheads, vec);
+  for (const void* q : ptrs) MVIT_REQUIRE(q && mvit_aligned16(q), "%s: null or unaligned pointer", who);
+  return MVIT_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mvit_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* cu_seqlens, int n_seg,
+                  int max_seqlen, int64_t total, int nheads, int head_dim, int64_t q_stride, int64_t k_stride,
+                  int64_t v_stride, int64_t o_stride, float scale, int dtype, mvit_stream_t stream) {
+  if (int rc = check_common("attn_fwd", cu_seqlens, n_seg, max_seqlen, total, nheads, head_dim, dtype,
+                            {q_stride, k_stride, v_stride, o_stride}, {q, k, v, o, (const void*)lse}))
+    return rc;
+  if (n_seg == 0 || max_seqlen == 0 || total == 0) return MVIT_OK;
+  AttnParams p = {};
+  p.q = q; p.k = k; p.v = v; p.out = o; p.lse = lse; p.cu = cu_seqlens; p.total = total; p.nheads = nheads;
+  p.q_stride = q_stride; p.k_stride = k_stride; p.v_stride = v_stride; p.o_stride = o_stride; p.scale = scale;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (dtype == MVIT_BF16) {
+    switch (head_dim) {
+      case 32: return launch_fwd_mfma<2>(p, n_seg, max_seqlen, s);
+      case 64: return launch_fwd_mfma<4>(p, n_seg, max_seqlen, s);
+      case 80: return launch_fwd_mfma<5>(p, n_seg, max_seqlen, s);
+      default: return launch_fwd_mfma<8>(p, n_seg, max_seqlen, s);
+    }
+  }
+  switch (head_dim) {
+    case 32: return launch_f32<32>(p, n_seg, max_seqlen, false, s);
+    case 64: return launch_f32<64>(p, n_seg, max_seqlen, false, s);
+    case 80: return launch_f32<80>(p, n_seg, max_seqlen, false, s);
+    default: return launch_f32<128>(p, n_seg, max_seqlen, false, s);
+  }
+}
+
+int mvit_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse, void* dq,
+                  void* dk, void* dv, float* delta, const int32_t* cu_seqlens, int n_seg, int max_seqlen, int64_t total,
+                  int nheads, int head_dim, int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
+                  int64_t do_stride, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride, float scale, int dtype,
+                  mvit_stream_t stream) {
+  if (int rc = check_common("attn_bwd", cu_seqlens, n_seg, max_seqlen, total, nheads, head_dim, dtype,
+                            {q_stride, k_stride, v_stride, o_stride, do_stride, dq_stride, dk_stride, dv_stride},
+                            {q, k, v, o, d_o, (const void*)lse, dq, dk, dv, (const void*)delta}))
+    return rc;
+  if (n_seg == 0 || max_seqlen == 0 || total == 0) return MVIT_OK;
+  AttnParams p = {};
+  p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.lse = const_cast<float*>(lse); p.delta = delta;
+  p.dq = dq; p.dk = dk; p.dv = dv; p.cu = cu_seqlens; p.total = total; p.nheads = nheads;
+  p.q_stride = q_stride; p.k_stride = k_stride; p.v_stride = v_stride; p.o_stride = o_stride; p.do_stride = do_stride;
+  p.dq_stride = dq_stride; p.dk_stride = dk_stride; p.dv_stride = dv_stride; p.scale = scale;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int64_t npairs = total * nheads;
+  const int dgrid = (int)((npairs + 255) / 256);
+  if (dtype == MVIT_BF16)
+    hipLaunchKernelGGL((attn_delta_kernel<bf16_t>), dgrid, 256, 0, s, (const bf16_t*)o, (const bf16_t*)d_o, delta, total, nheads, head_dim, o_stride, do_stride);
+  else
+    hipLaunchKernelGGL((attn_delta_kernel<float>), dgrid, 256, 0, s, (const float*)o, (const float*)d_o, delta, total, nheads, head_dim, o_stride, do_stride);
+  MVIT_CHECK_LAUNCH("attn_delta");
+  if (dtype == MVIT_BF16) {
+    switch (head_dim) {
+      case 32: return launch_bwd_mfma<2>(p, n_seg, max_seqlen, s);
+      case 64: return launch_bwd_mfma<4>(p, n_seg, max_seqlen, s);
+      case 80: return launch_bwd_mfma<5>(p, n_seg, max_seqlen, s);
+      default: return launch_bwd_mfma<8>(p, n_seg, max_seqlen, s);
+    }
+  }
+  switch (head_dim) {
+    case 32: return launch_f32<32>(p, n_seg, max_seqlen, true, s);
+    case 64: return launch_f32<64>(p, n_seg, max_seqlen, true, s);
+    case 80: return launch_f32<80>(p, n_seg, max_seqlen, true, s);
+    default: return launch_f32<128>(p, n_seg, max_seqlen, true, s);
+  }
+}
+
+}  // extern "C"

@@ -1,0 +1,83 @@
+"""ctypes binding of libmi355vit.so (the C ABI declared in include/mi355_vit.h).
+
+There is no fallback: if the shared library is missing or a call fails, a ``RuntimeError`` is raised.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libmi355vit.so"
+
+F32, BF16 = 0, 1
+
+EPI_NONE, EPI_BIAS, EPI_BIAS_RES, EPI_BIAS_GELU, EPI_SWIGLU, EPI_SWIGLU_BWD, EPI_GELU_BWD, EPI_ACCUM = range(8)
+
+_vp, _i64, _i32, _f32 = C.c_void_p, C.c_int64, C.c_int, C.c_float
+
+
+class GemmArgs(C.Structure):
+    _fields_ = [
+        ("dtype", _i32), ("out_dtype", _i32), ("trans_a", _i32), ("trans_b", _i32), ("epilogue", _i32), ("reserved", _i32),
+        ("M", _i64), ("N", _i64), ("K", _i64),
+        ("A", _vp), ("lda", _i64),
+        ("B", _vp), ("B2", _vp), ("ldb", _i64),
+        ("bias", _vp), ("bias2", _vp),
+        ("C", _vp), ("ldc", _i64),
+        ("R", _vp), ("ldr", _i64),
+        ("aux", _vp), ("ldaux", _i64), ("aux_off", _i64),
+    ]
+
+
+# name -> argument types (every function returns int except the two noted below)
+PROTOTYPES = {
+    "mvit_rot_pos_ids": [_vp, _i64, _i32, _vp],
+    "mvit_window_index": [_vp, _i64, _i32, _i32, _i32, _vp, _vp, _i64, _vp],
+    "mvit_cu_seqlens": [_vp, _i64, _vp, _i64, _vp],
+    "mvit_sp_token_cuts": [_i64, _i32, _vp],
+    "mvit_sp_window_cuts": [_i64, _i32, _vp, _i64, _vp, _vp],
+    "mvit_rmsnorm_fwd": [_vp, _vp, _vp, _vp, _i64, _i64, _f32, _i32, _vp],
+    "mvit_rmsnorm_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _i32, _vp],
+    "mvit_reduce_partials": [_vp, _i32, _i64, _vp, _i32, _vp],
+    "mvit_colsum": [_vp, _i64, _i64, _i64, _vp, _i32, _i32, _vp],
+    "mvit_rope": [_vp, _vp, _vp, _i64, _i32, _i32, _i64, _i32, _i32, _vp],
+    "mvit_gather_rows": [_vp, _vp, _vp, _i64, _i64, _vp],
+    "mvit_segment_copy": [_vp, _vp, _vp, _i64, _i64, _i64, _vp],
+    "mvit_pad_pack": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, C.c_uint32, _vp],
+    "mvit_cast2d": [_vp, _i64, _i32, _vp, _i64, _i32, _i64, _i64, _vp],
+    "mvit_gemm": [C.POINTER(GemmArgs), _vp],
+    "mvit_attn_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i64, _i32, _i32, _i64, _i64, _i64, _i64, _f32, _i32, _vp],
+    "mvit_attn_bwd": [_vp] * 11 + [_i32, _i32, _i64, _i32, _i32] + [_i64] * 8 + [_f32, _i32, _vp],
+}
+EXPORTS = sorted(list(PROTOTYPES) + ["mvit_version", "mvit_last_error"])
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load the library once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: the HIP extension has not been built "
+                "(run `python -c 'import __graft_entry__ as g; g.build()'`); there is no fallback path."
+            )
+        lib = C.CDLL(str(LIB_PATH))
+        for name, argtypes in PROTOTYPES.items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = C.c_int
+        lib.mvit_version.argtypes = []
+        lib.mvit_version.restype = C.c_int
+        lib.mvit_last_error.argtypes = []
+        lib.mvit_last_error.restype = C.c_char_p
+        _lib = lib
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().mvit_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{what} failed (code {rc}): {msg}")

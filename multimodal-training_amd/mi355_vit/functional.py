@@ -1,0 +1,284 @@
+"""Autograd functions of the vision tower.  Each one is a fixed sequence of C-ABI kernel launches with a
+hand-written backward (no autograd graph inside), so a transformer block is one node of PyTorch's graph.
+
+Reference spans (python/models/qwen2_5_vl/modeling_qwen2_5_vl.py):
+  VisionBlockFn   Qwen2_5_VLVisionBlock.forward :776-792 with _forward_standard :385-472 and the MLP :203-204
+  PatchEmbedFn    Qwen2_5_VisionPatchEmbed.forward :225-231
+  PermuteRowsFn   window reorder :934-937 and its inverse :1067-1068
+  MergerFn        Qwen2_5_VLPatchMerger.forward :260-262
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from . import _lib, ops
+
+E = _lib
+
+
+def round_up(v: int, m: int) -> int:
+    return (v + m - 1) // m * m
+
+
+@dataclass
+class BlockWeights:
+    """Compute-dtype operands of one block, laid out for the fused GEMMs.
+
+    wqkv [3C, C] / bqkv [3C]         q, k, v stacked
+    wgu  [2*Ipad, C] / bgu [2*Ipad]  gate rows [0, I), up rows [Ipad, Ipad+I); padding rows are zero
+    wdown [C, Ipad] / bdown [C]      padding columns are zero
+    """
+
+    norm1: torch.Tensor
+    norm2: torch.Tensor
+    wqkv: torch.Tensor
+    bqkv: torch.Tensor
+    wproj: torch.Tensor
+    bproj: torch.Tensor
+    wgu: torch.Tensor
+    bgu: torch.Tensor
+    wdown: torch.Tensor
+    bdown: torch.Tensor
+    C: int
+    I: int
+    Ipad: int
+
+
+# order of the parameter tensors handed to VisionBlockFn
+BLOCK_PARAM_ORDER = (
+    "norm1.weight", "norm2.weight",
+    "attn.q_proj.weight", "attn.q_proj.bias", "attn.k_proj.weight", "attn.k_proj.bias",
+    "attn.v_proj.weight", "attn.v_proj.bias", "attn.proj.weight", "attn.proj.bias",
+    "mlp.gate_proj.weight", "mlp.gate_proj.bias", "mlp.up_proj.weight", "mlp.up_proj.bias",
+    "mlp.down_proj.weight", "mlp.down_proj.bias",
+)
+
+
+def pack_block_weights(params: List[torch.Tensor], dtype: torch.dtype, into: Optional[BlockWeights]) -> BlockWeights:
+    """(Re)fill the packed operands from the 16 parameters (cast to `dtype` on the way)."""
+    (n1, n2, wq, bq, wk, bk, wv, bv, wp, bp, wg, bg, wu, bu, wd, bd) = params
+    C = wq.shape[1]
+    I = wg.shape[0]
+    Ipad = round_up(I, 8)
+    dev = wq.device
+    if into is None or into.wqkv.dtype != dtype or into.wqkv.device != dev:
+        z = lambda *s: torch.zeros(*s, dtype=dtype, device=dev)  # noqa: E731
+        into = BlockWeights(z(1, C), z(1, C), z(3 * C, C), z(1, 3 * C), z(C, C), z(1, C), z(2 * Ipad, C), z(1, 2 * Ipad),
+                            z(C, Ipad), z(1, C), C, I, Ipad)
+    cp = ops.cast2d
+    v = lambda t: t.detach().view(1, -1)  # noqa: E731
+    cp(v(n1), into.norm1)
+    cp(v(n2), into.norm2)
+    for j, (w, b) in enumerate(((wq, bq), (wk, bk), (wv, bv))):
+        cp(w.detach(), into.wqkv[j * C : (j + 1) * C])
+        cp(v(b), into.bqkv[:, j * C : (j + 1) * C])
+    cp(wp.detach(), into.wproj)
+    cp(v(bp), into.bproj)
+    for j, (w, b) in enumerate(((wg, bg), (wu, bu))):
+        cp(w.detach(), into.wgu[j * Ipad : j * Ipad + I])
+        cp(v(b), into.bgu[:, j * Ipad : j * Ipad + I])
+    cp(wd.detach(), into.wdown[:, :I])
+    cp(v(bd), into.bdown)
+    return into
+
+
+@dataclass
+class AttnGeometry:
+    """Per-layer attention layout: device cu_seqlens, the longest segment, head counts, rotary tables."""
+
+    cu: torch.Tensor
+    max_seqlen: int
+    nheads: int
+    head_dim: int
+    cos: torch.Tensor  # fp32 [S, head_dim]
+    sin: torch.Tensor
+
+
+def _block_forward(x: torch.Tensor, W: BlockWeights, geo: AttnGeometry, eps: float) -> Tuple[torch.Tensor, tuple]:
+    S, C = x.shape
+    H, hd = geo.nheads, geo.head_dim
+    n1, rstd1 = ops.rmsnorm_fwd(x, W.norm1.view(-1), eps)
+    qkv = torch.empty(S, 3 * C, dtype=x.dtype, device=x.device)
+    ops.gemm(n1, W.wqkv, qkv, epilogue=E.EPI_BIAS, bias=W.bqkv.view(-1))
+    ops.rope_(qkv, geo.cos, geo.sin, 2 * H, hd)  # q and k are the first 2*H heads of every row
+    o, lse = ops.attn_fwd(qkv[:, :C], qkv[:, C : 2 * C], qkv[:, 2 * C :], geo.cu, geo.max_seqlen, H, hd, hd**-0.5)
+    x1 = torch.empty_like(x)
+    ops.gemm(o, W.wproj, x1, epilogue=E.EPI_BIAS_RES, bias=W.bproj.view(-1), residual=x)
+    n2, rstd2 = ops.rmsnorm_fwd(x1, W.norm2.view(-1), eps)
+    gu = torch.empty(S, 2 * W.Ipad, dtype=x.dtype, device=x.device)
+    h = torch.empty(S, W.Ipad, dtype=x.dtype, device=x.device)
+    bgu = W.bgu.view(-1)
+    ops.gemm(n2, W.wgu[: W.Ipad], h, epilogue=E.EPI_SWIGLU, b2=W.wgu[W.Ipad :], bias=bgu[: W.Ipad], bias2=bgu[W.Ipad :],
+             aux=gu, aux_off=W.Ipad)
+    x2 = torch.empty_like(x)
+    ops.gemm(h, W.wdown, x2, epilogue=E.EPI_BIAS_RES, bias=W.bdown.view(-1), residual=x1)
+    return x2, (rstd1, n1, qkv, o, lse, x1, rstd2, n2, gu, h)
+
+
+def _block_backward(dx2: torch.Tensor, x: torch.Tensor, saved: tuple, W: BlockWeights, geo: AttnGeometry, gdt: Dict[str, torch.dtype]):
+    """Returns (dx, grads in BLOCK_PARAM_ORDER).  gdt maps parameter name -> gradient dtype."""
+    rstd1, n1, qkv, o, lse, x1, rstd2, n2, gu, h = saved
+    S, C = x.shape
+    H, hd = geo.nheads, geo.head_dim
+    I, Ipad = W.I, W.Ipad
+    dev = x.device
+    dx2 = dx2.contiguous()
+
+    # ---- MLP: x2 = x1 + down(silu(g) * u)
+    g_bd = ops.colsum(dx2, gdt["mlp.down_proj.bias"])
+    g_wd = torch.empty(C, I, dtype=gdt["mlp.down_proj.weight"], device=dev)
+    ops.gemm(dx2, h, g_wd, trans_a=True, trans_b=True, n=I)
+    dgu = torch.empty(S, 2 * Ipad, dtype=x.dtype, device=dev)
+    ops.gemm(dx2, W.wdown, dgu, trans_b=True, epilogue=E.EPI_SWIGLU_BWD, residual=gu, aux_off=Ipad)
+    g_bgu = ops.colsum(dgu, gdt["mlp.gate_proj.bias"])
+    g_wgu = torch.empty(2 * Ipad, C, dtype=gdt["mlp.gate_proj.weight"], device=dev)
+    ops.gemm(dgu, n2, g_wgu, trans_a=True, trans_b=True)
+    dn2 = torch.empty_like(x)
+    ops.gemm(dgu, W.wgu, dn2, trans_b=True)
+    del dgu
+    dx1, g_n2 = ops.rmsnorm_bwd(dn2, x1, W.norm2.view(-1), rstd2, dx_add=dx2, w_grad_dtype=gdt["norm2.weight"])
+
+    # ---- attention: x1 = x + proj(attn(rope(qkv(norm1(x)))))
+    g_bp = ops.colsum(dx1, gdt["attn.proj.bias"])
+    g_wp = torch.empty(C, C, dtype=gdt["attn.proj.weight"], device=dev)
+    ops.gemm(dx1, o, g_wp, trans_a=True, trans_b=True)
+    d_o = dn2  # reuse the buffer
+    ops.gemm(dx1, W.wproj, d_o, trans_b=True)
+    dqkv = torch.empty_like(qkv)
+    ops.attn_bwd(qkv[:, :C], qkv[:, C : 2 * C], qkv[:, 2 * C :], o, d_o, lse, geo.cu, geo.max_seqlen, H, hd, hd**-0.5,
+                 dqkv[:, :C], dqkv[:, C : 2 * C], dqkv[:, 2 * C :])
+    ops.rope_(dqkv, geo.cos, geo.sin, 2 * H, hd, backward=True)
+    g_bqkv = ops.colsum(dqkv, gdt["attn.q_proj.bias"])
+    g_wqkv = torch.empty(3 * C, C, dtype=gdt["attn.q_proj.weight"], device=dev)
+    ops.gemm(dqkv, n1, g_wqkv, trans_a=True, trans_b=True)
+    dn1 = d_o
+    ops.gemm(dqkv, W.wqkv, dn1, trans_b=True)
+    dx, g_n1 = ops.rmsnorm_bwd(dn1, x, W.norm1.view(-1), rstd1, dx_add=dx1, w_grad_dtype=gdt["norm1.weight"])
+
+    grads = (
+        g_n1, g_n2,
+        g_wqkv[:C], g_bqkv[:C], g_wqkv[C : 2 * C], g_bqkv[C : 2 * C], g_wqkv[2 * C :], g_bqkv[2 * C :],
+        g_wp, g_bp,
+        g_wgu[:I], g_bgu[:I], g_wgu[Ipad : Ipad + I], g_bgu[Ipad : Ipad + I],
+        g_wd, g_bd,
+    )
+    return dx, grads
+
+
+class VisionBlockFn(torch.autograd.Function):
+    """One transformer block.  With `checkpoint` only the block input is kept and the forward is re-run in
+    the backward (the native counterpart of torch.utils.checkpoint around the block, [tf] modeling_layers.py:79)."""
+
+    @staticmethod
+    def forward(ctx, x, holder, geo: AttnGeometry, eps: float, checkpoint: bool, *params):
+        W = holder.packed(x.dtype)
+        x = x.contiguous()
+        x2, saved = _block_forward(x, W, geo, eps)
+        ctx.holder, ctx.geo, ctx.eps, ctx.checkpoint = holder, geo, eps, checkpoint
+        ctx.gdt = {name: p.dtype for name, p in zip(BLOCK_PARAM_ORDER, params)}
+        ctx.x = x
+        ctx.saved = None if checkpoint else saved
+        return x2
+
+    @staticmethod
+    def backward(ctx, dx2):
+        x, geo = ctx.x, ctx.geo
+        W = ctx.holder.packed(x.dtype)
+        saved = ctx.saved
+        if saved is None:
+            _, saved = _block_forward(x, W, geo, ctx.eps)
+        dx, grads = _block_backward(dx2, x, saved, W, geo, ctx.gdt)
+        ctx.saved = None
+        ctx.x = None
+        return (dx, None, None, None, None) + tuple(grads)
+
+
+class PatchEmbedFn(torch.autograd.Function):
+    """[S, 1176] pixels x Conv3d weight viewed as [C, 1176]: a GEMM without bias."""
+
+    @staticmethod
+    def forward(ctx, pixels, weight, compute_dtype):
+        w2 = weight.detach().reshape(weight.shape[0], -1)
+        K = w2.shape[1]
+        px = pixels.detach().reshape(-1, K)
+        if px.dtype != compute_dtype or not px.is_contiguous():
+            px = ops.cast2d(px if px.stride(1) == 1 else px.contiguous(), torch.empty(px.shape, dtype=compute_dtype, device=px.device))
+        if w2.dtype != compute_dtype:
+            w2 = ops.cast2d(w2, torch.empty(w2.shape, dtype=compute_dtype, device=w2.device))
+        out = torch.empty(px.shape[0], w2.shape[0], dtype=compute_dtype, device=px.device)
+        ops.gemm(px, w2, out)
+        ctx.px, ctx.wshape, ctx.wdtype = px, weight.shape, weight.dtype
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        px = ctx.px
+        gw = torch.empty(dout.shape[1], px.shape[1], dtype=ctx.wdtype, device=px.device)
+        ops.gemm(dout.contiguous(), px, gw, trans_a=True, trans_b=True)
+        return None, gw.view(ctx.wshape), None
+
+
+class PermuteRowsFn(torch.autograd.Function):
+    """out.view(n, unit*cols)[i] = x.view(n, unit*cols)[index[i]]; `inverse` is the inverse permutation."""
+
+    @staticmethod
+    def forward(ctx, x, index, inverse, unit):
+        ctx.inverse, ctx.unit = inverse, unit
+        return ops.gather_rows(x.contiguous(), index, unit)
+
+    @staticmethod
+    def backward(ctx, dout):
+        return ops.gather_rows(dout.contiguous(), ctx.inverse, ctx.unit), None, None, None
+
+
+def _as_dtype(t: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    t = t.detach()
+    if t.dtype == dtype and t.is_contiguous():
+        return t
+    t2 = t.reshape(1, -1) if t.dim() == 1 else t
+    out = ops.cast2d(t2.contiguous() if t2.stride(-1) != 1 else t2, torch.empty(t2.shape, dtype=dtype, device=t.device))
+    return out.view(t.shape)
+
+
+class MergerFn(torch.autograd.Function):
+    """RMSNorm(C) -> view [S/unit, unit*C] -> Linear + exact GELU -> Linear."""
+
+    @staticmethod
+    def forward(ctx, x, ln_w, w0, b0, w2, b2, unit, eps):
+        T = x.dtype
+        x = x.contiguous()
+        lw, W0, B0, W2, B2 = (_as_dtype(t, T) for t in (ln_w, w0, b0, w2, b2))
+        ln, rstd = ops.rmsnorm_fwd(x, lw, eps)
+        M = x.shape[0] // unit
+        ln2 = ln.view(M, -1)
+        z = torch.empty(M, W0.shape[0], dtype=T, device=x.device)
+        y1 = torch.empty_like(z)
+        ops.gemm(ln2, W0, y1, epilogue=E.EPI_BIAS_GELU, bias=B0, aux=z)
+        y2 = torch.empty(M, W2.shape[0], dtype=T, device=x.device)
+        ops.gemm(y1, W2, y2, epilogue=E.EPI_BIAS, bias=B2)
+        ctx.saved = (x, lw, rstd, ln2, z, y1, W0, W2)
+        ctx.gdt = (ln_w.dtype, w0.dtype, b0.dtype, w2.dtype, b2.dtype)
+        return y2
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, lw, rstd, ln2, z, y1, W0, W2 = ctx.saved
+        ctx.saved = None
+        dy = dy.contiguous()
+        dev = x.device
+        g_b2 = ops.colsum(dy, ctx.gdt[4])
+        g_w2 = torch.empty(W2.shape, dtype=ctx.gdt[3], device=dev)
+        ops.gemm(dy, y1, g_w2, trans_a=True, trans_b=True)
+        dz = torch.empty_like(z)
+        ops.gemm(dy, W2, dz, trans_b=True, epilogue=E.EPI_GELU_BWD, residual=z)
+        g_b0 = ops.colsum(dz, ctx.gdt[2])
+        g_w0 = torch.empty(W0.shape, dtype=ctx.gdt[1], device=dev)
+        ops.gemm(dz, ln2, g_w0, trans_a=True, trans_b=True)
+        dln = torch.empty_like(ln2)
+        ops.gemm(dz, W0, dln, trans_b=True)
+        dx, g_ln = ops.rmsnorm_bwd(dln.view(x.shape), x, lw, rstd, w_grad_dtype=ctx.gdt[0])
+        return dx, g_ln, g_w0, g_b0, g_w2, g_b2, None, None
