@@ -96,14 +96,30 @@ __device__ __forceinline__ void load_rowfrag_lds(RowFrag<ND>& f, const bf16_t* t
   for (int ks = 0; ks < G::NK32; ++ks) f.k32[ks] = *reinterpret_cast<const bf16x8*>(p + 32 * ks + 8 * g);
   if (G::TAIL16) f.k16 = *reinterpret_cast<const bf16x4*>(p + 32 * G::NK32 + 4 * g);
 }
-// acc += rows(a) . rows(b)^T over head_dim  (16x16 tile)
+// acc = rows(a) . rows(b)^T over head_dim  (16x16 tile).
+// The 16-wide remainder of head_dim (odd ND) is issued as a 32-wide MFMA whose upper four contraction slots
+// are zero: a v_mfma_f32_16x16x16_bf16 chained onto the accumulator of the 32-wide steps returned wrong sums
+// on gfx950 (also with an all-zero remainder), so that instruction is not used here.
+#ifndef MVIT_TAIL_MODE
+#define MVIT_TAIL_MODE 0
+#endif
 template <int ND>
 __device__ __forceinline__ f32x4 dot_frag(const RowFrag<ND>& a, const RowFrag<ND>& b) {
   using G = Geo<ND>;
   f32x4 c = {0.f, 0.f, 0.f, 0.f};
+#if MVIT_TAIL_MODE == 1
+  if (G::TAIL16) c = mfma16(a.k16, b.k16, c);
+#endif
 #pragma unroll
   for (int ks = 0; ks < G::NK32; ++ks) c = mfma32(a.k32[ks], b.k32[ks], c);
-  if (G::TAIL16) c = mfma16(a.k16, b.k16, c);
+#if MVIT_TAIL_MODE == 0
+  if (G::TAIL16) {
+    const bf16_t z = (bf16_t)0.f;
+    const bf16x8 ax = {a.k16[0], a.k16[1], a.k16[2], a.k16[3], z, z, z, z};
+    const bf16x8 bx = {b.k16[0], b.k16[1], b.k16[2], b.k16[3], z, z, z, z};
+    c = mfma32(ax, bx, c);
+  }
+#endif
   return c;
 }
 

@@ -1,0 +1,379 @@
+"""Parity of every HIP kernel (called through the C ABI) against the CPU oracle.
+
+Tolerances (max |a-b| / max |b|): 1e-4 in fp32, 2e-2 in bf16; index / copy kernels are bit-exact.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import sp_oracle, vit_oracle
+from oracle.vit_oracle import max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-2}
+DEV = "cuda:0"
+
+
+def _ops():
+    from mi355_vit import ops
+
+    return ops
+
+
+def _rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+def _announce(msg):
+    print(f"[case] {msg}", flush=True)
+
+
+# ------------------------------------------------------------------------------------------ RMSNorm
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,cols", [(512, 1280), (37, 256), (5, 100), (4096, 1280)])
+def test_rmsnorm_fwd_bwd(dtype, rows, cols):
+    _announce(f"rmsnorm {dtype} {rows}x{cols}")
+    ops = _ops()
+    x = _rand((rows, cols), dtype, 0)
+    w = (1.0 + 0.1 * _rand((cols,), torch.float32, 1)).to(dtype)
+    dy = _rand((rows, cols), dtype, 2)
+    add = _rand((rows, cols), dtype, 3)
+    y, rstd = ops.rmsnorm_fwd(x.to(DEV), w.to(DEV), 1e-6)
+    xr = x.float().requires_grad_(True)
+    wr = w.float().requires_grad_(True)
+    yr = vit_oracle.rms_norm(xr, wr, 1e-6)
+    # the oracle formula itself is pinned against the library routine
+    assert max_rel_err(yr, F.rms_norm(xr, (cols,), wr, 1e-6)) < 1e-6
+    assert max_rel_err(y, yr) < TOL[dtype]
+    yr.backward(dy.float())
+    dx, dw = ops.rmsnorm_bwd(dy.to(DEV), x.to(DEV), w.to(DEV), rstd, dx_add=add.to(DEV))
+    assert max_rel_err(dx, xr.grad + add.float()) < TOL[dtype]
+    assert max_rel_err(dw, wr.grad) < TOL[dtype]
+    dx2, _ = ops.rmsnorm_bwd(dy.to(DEV), x.to(DEV), w.to(DEV), rstd)
+    assert max_rel_err(dx2, xr.grad) < TOL[dtype]
+
+
+# ------------------------------------------------------------------------------------------ RoPE
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("S,H,d", [(300, 16, 80), (64, 8, 32), (17, 4, 6)])
+def test_rope_fwd_bwd(dtype, S, H, d):
+    _announce(f"rope {dtype} S={S} H={H} d={d}")
+    ops = _ops()
+    pad = 8 if d % 8 == 0 else 0
+    x = _rand((S, H * d + pad * d), dtype, 0)  # extra columns must stay untouched
+    ang = _rand((S, d), torch.float32, 1, 3.0)  # deliberately different halves: the general form
+    cos, sin = ang.cos(), ang.sin()
+    xg = x.to(DEV).clone()
+    ops.rope_(xg, cos.to(DEV), sin.to(DEV), H, d)
+    ref = vit_oracle.rope_apply(x[:, : H * d].reshape(S, H, d), cos, sin).reshape(S, H * d)
+    assert max_rel_err(xg[:, : H * d], ref.float()) < TOL[dtype]
+    assert torch.equal(xg[:, H * d :].cpu(), x[:, H * d :])
+    # closed form: every (j, j+d/2) pair is rotated when both halves share the angle -> norms are preserved
+    a2 = torch.cat([ang[:, : d // 2]] * 2, dim=-1)
+    xf = _rand((S, H * d), torch.float32, 5)
+    xr = xf.to(DEV).clone()
+    ops.rope_(xr, a2.cos().to(DEV), a2.sin().to(DEV), H, d)
+    n0 = xf.view(S, H, 2, d // 2).pow(2).sum(2)
+    n1 = xr.cpu().view(S, H, 2, d // 2).pow(2).sum(2)
+    assert torch.allclose(n0, n1, rtol=1e-4, atol=1e-5)
+    # backward = transpose of the forward map
+    xin = x[:, : H * d].float().reshape(S, H, d).requires_grad_(True)
+    g = _rand((S, H * d), dtype, 7)
+    vit_oracle.rope_apply(xin, cos, sin).backward(g.float().reshape(S, H, d))
+    gg = g.to(DEV).clone()
+    ops.rope_(gg, cos.to(DEV), sin.to(DEV), H, d, backward=True)
+    assert max_rel_err(gg, xin.grad.reshape(S, H * d)) < TOL[dtype]
+
+
+# ------------------------------------------------------------------------------------------ copies
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gather_rows_window_permutation_bit_exact(dtype):
+    ops = _ops()
+    grid = torch.tensor([[1, 18, 22], [2, 8, 12], [1, 16, 16]])
+    widx, cu = ops.window_index(grid, 2, 112, 14)
+    S = int((grid[:, 0] * grid[:, 1] * grid[:, 2]).sum())
+    x = _rand((S, 1280), dtype, 0)
+    out = ops.gather_rows(x.to(DEV), widx.to(DEV), 4).cpu()
+    ref = x.view(S // 4, 4, -1)[widx].reshape(S, -1)
+    assert torch.equal(out.view(torch.int16 if dtype == torch.bfloat16 else torch.int32), ref.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+    rev = torch.argsort(widx)
+    back = ops.gather_rows(out.to(DEV), rev.to(DEV), 4).cpu()
+    assert torch.equal(back.view(torch.int32 if dtype == torch.float32 else torch.int16), x.view(torch.int32 if dtype == torch.float32 else torch.int16))
+    # odd row width (falls back to 4-byte words)
+    y = _rand((12, 6), dtype, 1)
+    perm = torch.randperm(12, generator=torch.Generator().manual_seed(0))
+    assert torch.equal(ops.gather_rows(y.to(DEV), perm.to(DEV)).cpu(), y[perm])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sp", [1, 2, 3, 4, 8])
+def test_split_gather_bit_exact(dtype, sp):
+    """split_pack_by_sp for every rank, then the re-interleave: must reproduce the input bit for bit."""
+    from mi355_vit import sequence_parallel_utils as spu
+
+    ops = _ops()
+    g = torch.Generator().manual_seed(2)
+    hw = 2 * torch.randint(4, 20, (5, 2), generator=g)
+    grid = torch.cat([torch.ones(5, 1, dtype=torch.long), hw], dim=1)
+    grid[1, 0] = 2
+    _, cu_w = ops.window_index(grid, 2, 112, 14)
+    lengths = (ops.cu_seqlens(grid)[1:] - ops.cu_seqlens(grid)[:-1]).tolist()
+    S = sum(lengths)
+    x = _rand((S, 320), dtype, 3)
+    xg = x.to(DEV)
+    for windows in (None, cu_w):
+        packs, metas = [], []
+        for r in range(sp):
+            pk, meta = spu.split_pack_by_sp(xg, lengths, r, sp, cu_window_seqlens=windows)
+            ref = sp_oracle.split_rows(x.view(torch.int16 if dtype == torch.bfloat16 else torch.int32).numpy(), lengths, r, sp,
+                                       None if windows is None else windows.tolist())
+            assert np.array_equal(pk.cpu().view(torch.int16 if dtype == torch.bfloat16 else torch.int32).numpy(), ref)
+            packs.append(pk)
+            metas.append(meta)
+        lm = [m.local_lengths for m in metas]
+        rebuilt = spu.gather_rank_packs(packs, lm)
+        assert torch.equal(rebuilt.cpu().view(torch.uint8), x.view(torch.uint8))
+        assert sum(m.total_local_len for m in metas) == S
+
+
+def test_split_gather_reference_sizes():
+    """tests/test_split_gather.py of the reference: arange tensors of 1024 and 1020 rows x 1280, two ranks."""
+    from mi355_vit import sequence_parallel_utils as spu
+
+    for rows in (1024, 1020):
+        x = torch.arange(rows * 1280, dtype=torch.float32).reshape(rows, 1280).to(DEV)
+        packs, lm = [], []
+        for r in range(2):
+            pk, meta = spu.split_pack_by_sp(x, [rows], r, 2)
+            packs.append(pk)
+            lm.append(meta.local_lengths)
+        assert packs[0].shape[0] == rows // 2
+        assert torch.equal(packs[0], x[: rows // 2])
+        assert torch.equal(spu.gather_rank_packs(packs, lm), x)
+
+
+def test_pad_unpad_and_local_rope():
+    from mi355_vit import sequence_parallel_utils as spu
+
+    x = _rand((20, 64), torch.bfloat16, 0).to(DEV)
+    pk, meta = spu.split_pack_by_sp(x, [12, 8], 0, 2)
+    assert meta.local_lengths == [6, 4]
+    padded, mask = spu.pad_pack_to_batch(pk, meta, pad_value=-999.0)
+    assert padded.shape == (2, 6, 64) and mask.dtype == torch.bool
+    assert mask[0].all() and mask[1, :4].all() and not mask[1, 4:].any()
+    assert (padded[1, 4:] == -999.0).all()
+    pad_bf16 = torch.tensor(-999.0, dtype=torch.bfloat16).float().item()  # the pad value as bf16 stores it
+    ref, rmask = sp_oracle.pad_rows(pk.cpu().float().numpy(), [6, 4], pad_value=pad_bf16)
+    assert np.array_equal(padded.cpu().float().numpy(), ref) and np.array_equal(mask.cpu().numpy(), rmask)
+    back, lens = spu.unpad_batch_to_pack(padded, mask, return_lengths=True)
+    assert lens == [6, 4] and torch.equal(back, pk)
+    p2, m2 = spu.pad_pack_to_batch(pk, meta, pad_to=9, enforce_min_pad=1)
+    assert p2.shape == (2, 9, 64)
+    with pytest.raises(ValueError):
+        spu.pad_pack_to_batch(pk, meta, pad_to=3)
+    empty, _ = spu.unpad_batch_to_pack(torch.randn(2, 5, 32, device=DEV), torch.zeros(2, 5, dtype=torch.bool, device=DEV))
+    assert empty.shape == (0, 32)
+    cos, sin = torch.randn(20, 32, device=DEV), torch.randn(20, 32, device=DEV)
+    c0, s0, m0 = spu.build_local_rope(meta, cos, sin)
+    assert m0 is None and torch.equal(c0[:6], cos[0:6]) and torch.equal(c0[6:10], cos[12:16]) and torch.equal(s0[6:], sin[12:16])
+    cp, sp_, mk = spu.build_local_rope(meta, cos, sin, pad_to=7)
+    assert cp.shape == (2, 7, 32) and mk.shape == (2, 7) and (cp[1, 4:] == 0).all() and torch.equal(cp[0, :6], cos[:6])
+
+
+def test_cast2d_and_colsum():
+    ops = _ops()
+    x = _rand((300, 70), torch.float32, 0)
+    dst = torch.zeros(300, 96, dtype=torch.bfloat16, device=DEV)
+    ops.cast2d(x.to(DEV), dst[:, 8:78])
+    assert torch.equal(dst[:, 8:78].cpu(), x.to(torch.bfloat16)) and (dst[:, :8] == 0).all() and (dst[:, 78:] == 0).all()
+    for dtype in (torch.float32, torch.bfloat16):
+        y = _rand((1000, 130), dtype, 1)
+        s = ops.colsum(y.to(DEV)[:, 1:129], torch.float32)
+        assert max_rel_err(s, y[:, 1:129].float().sum(0)) < 1e-5
+
+
+# ------------------------------------------------------------------------------------------ GEMM
+def _gemm_ref(a, b):
+    return a.double() @ b.double().t()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(512, 1280, 1280), (300, 200, 72), (1000, 3424, 1280), (260, 1280, 1176), (8, 8, 8)])
+def test_gemm_plain_bias_residual(dtype, M, N, K):
+    _announce(f"gemm NT {dtype} {M}x{N}x{K}")
+    ops = _ops()
+    from mi355_vit import _lib as E
+
+    a, b = _rand((M, K), dtype, 0), _rand((N, K), dtype, 1, K**-0.5)
+    bias, res = _rand((N,), dtype, 2), _rand((M, N), dtype, 3)
+    ref = _gemm_ref(a, b)
+    out = torch.empty(M, N, dtype=dtype, device=DEV)
+    ops.gemm(a.to(DEV), b.to(DEV), out)
+    assert max_rel_err(out, ref) < TOL[dtype]
+    ops.gemm(a.to(DEV), b.to(DEV), out, epilogue=E.EPI_BIAS, bias=bias.to(DEV))
+    assert max_rel_err(out, ref + bias.double()) < TOL[dtype]
+    ops.gemm(a.to(DEV), b.to(DEV), out, epilogue=E.EPI_BIAS_RES, bias=bias.to(DEV), residual=res.to(DEV))
+    assert max_rel_err(out, ref + bias.double() + res.double()) < TOL[dtype]
+    ops.gemm(a.to(DEV), b.to(DEV), out, epilogue=E.EPI_ACCUM)
+    assert max_rel_err(out, 2 * ref + bias.double() + res.double()) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(512, 1280, 3840), (300, 200, 72), (130, 1280, 6848), (257, 3420, 1280)])
+def test_gemm_dgrad_layout(dtype, M, N, K):
+    """C = A . W with W stored [K, N] (the weight as it lies in memory): trans_b."""
+    _announce(f"gemm NN {dtype} {M}x{N}x{K}")
+    ops = _ops()
+    a, w = _rand((M, K), dtype, 0), _rand((K, (N + 7) // 8 * 8), dtype, 1, K**-0.5)
+    out = torch.empty(M, N, dtype=dtype, device=DEV)
+    ops.gemm(a.to(DEV), w.to(DEV), out, trans_b=True, n=N)
+    assert max_rel_err(out, a.double() @ w.double()[:, :N]) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype,odt", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("S,No,Ni", [(1000, 1280, 1280), (515, 3840, 256), (70, 6848, 1280), (2052, 1280, 3420)])
+def test_gemm_wgrad_layout(dtype, odt, S, No, Ni):
+    """dW[No, Ni] = dY^T . X with dY [S, No] and X [S, Ni] as they lie in memory: trans_a and trans_b."""
+    _announce(f"gemm TT {dtype}->{odt} S={S} {No}x{Ni}")
+    ops = _ops()
+    ldx = (Ni + 7) // 8 * 8
+    dy, x = _rand((S, No), dtype, 0), _rand((S, ldx), dtype, 1)
+    out = torch.empty(No, Ni, dtype=odt, device=DEV)
+    ops.gemm(dy.to(DEV), x.to(DEV), out, trans_a=True, trans_b=True, n=Ni)
+    assert max_rel_err(out, dy.double().t() @ x.double()[:, :Ni]) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gemm_gelu_and_swiglu_epilogues(dtype):
+    ops = _ops()
+    from mi355_vit import _lib as E
+
+    M, K, N = 384, 640, 520
+    a = _rand((M, K), dtype, 0)
+    w, b = _rand((N, K), dtype, 1, K**-0.5), _rand((N,), dtype, 2)
+    z = torch.empty(M, N, dtype=dtype, device=DEV)
+    y = torch.empty_like(z)
+    ops.gemm(a.to(DEV), w.to(DEV), y, epilogue=E.EPI_BIAS_GELU, bias=b.to(DEV), aux=z)
+    zr = F.linear(a.float(), w.float(), b.float())
+    assert max_rel_err(z, zr) < TOL[dtype]
+    assert max_rel_err(y, F.gelu(z.float().cpu())) < TOL[dtype]  # gelu of the stored pre-activation
+    # gelu backward epilogue: dz = (dy . W2) * gelu'(z)
+    O = 264
+    dy, w2 = _rand((M, O), dtype, 3), _rand((O, N), dtype, 4, N**-0.5)
+    dz = torch.empty(M, N, dtype=dtype, device=DEV)
+    ops.gemm(dy.to(DEV), w2.to(DEV), dz, trans_b=True, epilogue=E.EPI_GELU_BWD, residual=z)
+    zc = z.float().cpu().requires_grad_(True)
+    F.gelu(zc).backward(dy.float() @ w2.float())
+    assert max_rel_err(dz, zc.grad) < TOL[dtype]
+
+    # SwiGLU: packed [2*Ipad, K] weight with zero padding rows, as the block uses it
+    I, Ipad = 516, 520
+    wg, wu = _rand((I, K), dtype, 5, K**-0.5), _rand((I, K), dtype, 6, K**-0.5)
+    bg, bu = _rand((I,), dtype, 7), _rand((I,), dtype, 8)
+    wgu = torch.zeros(2 * Ipad, K, dtype=dtype)
+    wgu[:I], wgu[Ipad : Ipad + I] = wg, wu
+    bgu = torch.zeros(2 * Ipad, dtype=dtype)
+    bgu[:I], bgu[Ipad : Ipad + I] = bg, bu
+    wgu, bgu = wgu.to(DEV), bgu.to(DEV)
+    gu = torch.full((M, 2 * Ipad), float("nan"), dtype=dtype, device=DEV)
+    h = torch.full((M, Ipad), float("nan"), dtype=dtype, device=DEV)
+    ops.gemm(a.to(DEV), wgu[:Ipad], h, epilogue=E.EPI_SWIGLU, b2=wgu[Ipad:], bias=bgu[:Ipad], bias2=bgu[Ipad:], aux=gu, aux_off=Ipad)
+    gr, ur = F.linear(a.float(), wg.float(), bg.float()), F.linear(a.float(), wu.float(), bu.float())
+    assert max_rel_err(gu[:, :I], gr) < TOL[dtype] and max_rel_err(gu[:, Ipad : Ipad + I], ur) < TOL[dtype]
+    assert max_rel_err(h[:, :I], F.silu(gr) * ur) < TOL[dtype]
+    assert (h[:, I:] == 0).all() and (gu[:, I:Ipad] == 0).all() and (gu[:, Ipad + I :] == 0).all()
+    # backward epilogue: (dg, du) from dh = dx . Wdown, Wdown stored [C, Ipad] with zero padding columns
+    Cc = 256
+    dx, wd = _rand((M, Cc), dtype, 9), torch.zeros(Cc, Ipad, dtype=dtype)
+    wd[:, :I] = _rand((Cc, I), dtype, 10, I**-0.5)
+    dgu = torch.full((M, 2 * Ipad), float("nan"), dtype=dtype, device=DEV)
+    ops.gemm(dx.to(DEV), wd.to(DEV), dgu, trans_b=True, epilogue=E.EPI_SWIGLU_BWD, residual=gu, aux_off=Ipad)
+    g0 = gu[:, :I].float().cpu().requires_grad_(True)
+    u0 = gu[:, Ipad : Ipad + I].float().cpu().requires_grad_(True)
+    (F.silu(g0) * u0).backward(dx.float() @ wd.float()[:, :I])
+    assert max_rel_err(dgu[:, :I], g0.grad) < TOL[dtype] and max_rel_err(dgu[:, Ipad : Ipad + I], u0.grad) < TOL[dtype]
+    assert (dgu[:, I:Ipad] == 0).all() and (dgu[:, Ipad + I :] == 0).all()
+
+
+# ------------------------------------------------------------------------------------------ attention
+def _attn_case(dtype, seglens, H, d, seed=0, qkv_packed=True):
+    ops = _ops()
+    S = sum(seglens)
+    cu = torch.tensor([0] + list(np.cumsum(seglens)), dtype=torch.int32)
+    if qkv_packed:  # q, k, v are column blocks of one [S, 3*H*d] buffer, as in the block
+        qkv = _rand((S, 3 * H * d), dtype, seed)
+        q, k, v = qkv[:, : H * d], qkv[:, H * d : 2 * H * d], qkv[:, 2 * H * d :]
+        qkvg = qkv.to(DEV)
+        qg, kg, vg = qkvg[:, : H * d], qkvg[:, H * d : 2 * H * d], qkvg[:, 2 * H * d :]
+    else:
+        q, k, v = (_rand((S, H * d), dtype, seed + i) for i in range(3))
+        qg, kg, vg = q.to(DEV), k.to(DEV), v.to(DEV)
+    do = _rand((S, H * d), dtype, seed + 7)
+    scale = d**-0.5
+    og, lse = ops.attn_fwd(qg, kg, vg, cu.to(DEV), max(seglens), H, d, scale)
+    qr, kr, vr = (t.float().reshape(S, H, d).clone().requires_grad_(True) for t in (q, k, v))
+    oref = vit_oracle.attention(qr, kr, vr, cu)
+    # pin the oracle's attention against the library routine on the first segment
+    L0 = seglens[0]
+    if L0:
+        sd = F.scaled_dot_product_attention(qr[:L0].transpose(0, 1)[None], kr[:L0].transpose(0, 1)[None], vr[:L0].transpose(0, 1)[None])
+        assert max_rel_err(oref[:L0], sd[0].transpose(0, 1)) < 1e-5
+    assert max_rel_err(og, oref.reshape(S, H * d)) < TOL[dtype], "forward"
+    lse_ref = []
+    for a, b in zip(cu[:-1].tolist(), cu[1:].tolist()):
+        s = torch.einsum("qhd,khd->hqk", qr[a:b], kr[a:b]) * scale
+        lse_ref.append(torch.logsumexp(s, dim=-1))
+    assert torch.allclose(lse.cpu(), torch.cat(lse_ref, dim=1).detach(), rtol=2e-3 if dtype == torch.bfloat16 else 1e-5, atol=2e-3 if dtype == torch.bfloat16 else 1e-5)
+    oref.backward(do.float().reshape(S, H, d))
+    dq, dk, dv = (torch.empty(S, H * d, dtype=dtype, device=DEV) for _ in range(3))
+    ops.attn_bwd(qg, kg, vg, og, do.to(DEV), lse, cu.to(DEV), max(seglens), H, d, scale, dq, dk, dv)
+    for name, got, ref in (("dq", dq, qr.grad), ("dk", dk, kr.grad), ("dv", dv, vr.grad)):
+        assert max_rel_err(got, ref.reshape(S, H * d)) < TOL[dtype], name
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize(
+    "seglens,H,d",
+    [
+        ([64] * 6, 16, 80),  # windows
+        ([64, 16, 48, 64, 32, 4], 4, 80),  # ragged edge windows
+        ([256, 256], 16, 80),  # cfg-1 full layer
+        ([300, 77, 1, 130], 2, 80),  # ragged, single-token segment
+        ([100, 60], 8, 32),
+        ([129], 2, 64),
+        ([96, 200], 2, 128),
+    ],
+)
+def test_attention_fwd_bwd(dtype, seglens, H, d):
+    _announce(f"attention {dtype} seglens={seglens} H={H} d={d}")
+    _attn_case(dtype, seglens, H, d)
+
+
+def test_attention_long_segment_bf16():
+    """One 2,048-token segment with 4 heads (the sequence-parallel share shape, scaled down)."""
+    _announce("attention bf16 long")
+    _attn_case(torch.bfloat16, [2048, 1000], 4, 80, qkv_packed=False)
+
+
+def test_attention_softmax_invariants():
+    """Properties that hold at any size: V constant -> O constant; outputs independent across segments."""
+    ops = _ops()
+    S, H, d = 700, 4, 80
+    cu = torch.tensor([0, 300, 700], dtype=torch.int32, device=DEV)
+    q, k = (_rand((S, H * d), torch.bfloat16, i).to(DEV) for i in range(2))
+    v = torch.ones(S, H * d, dtype=torch.bfloat16, device=DEV) * 0.5
+    o, _ = ops.attn_fwd(q, k, v, cu, 400, H, d, d**-0.5)
+    assert torch.allclose(o.float(), torch.full_like(o.float(), 0.5), atol=4e-3)
+    v2 = _rand((S, H * d), torch.bfloat16, 5).to(DEV)
+    o1, _ = ops.attn_fwd(q, k, v2, cu, 400, H, d, d**-0.5)
+    k2, v3 = k.clone(), v2.clone()
+    k2[300:] = 0
+    v3[300:] = 1
+    o2, _ = ops.attn_fwd(q, k2, v3, cu, 400, H, d, d**-0.5)
+    assert torch.equal(o1[:300], o2[:300])

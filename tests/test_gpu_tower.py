@@ -1,0 +1,187 @@
+"""End-to-end parity of the vision tower (forward, every parameter gradient) against the CPU oracle, and the
+VisionTrainer step API on the GPU."""
+
+import copy
+
+import pytest
+import torch
+
+from oracle import vit_oracle
+from oracle.vit_oracle import OracleConfig, max_rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _build(cfg_kwargs, seed, dtype):
+    from mi355_vit.config import Qwen2_5_VLVisionConfig
+    from mi355_vit.modeling import Qwen2_5_VisionTransformerPretrainedModel
+
+    torch.manual_seed(seed)
+    model = Qwen2_5_VisionTransformerPretrainedModel(Qwen2_5_VLVisionConfig(**cfg_kwargs))
+    model.to(dtype)
+    return model
+
+
+def _oracle_cfg(kw):
+    return OracleConfig(**{k: v for k, v in kw.items() if k in OracleConfig.__dataclass_fields__})
+
+
+def _oracle_run(model_cpu, kw, pixels, grid, gout):
+    """fp32 oracle forward/backward on the (possibly bf16-rounded) weights of `model_cpu`."""
+    params = {k: v.detach().float().clone().requires_grad_(True) for k, v in model_cpu.state_dict().items()}
+    inv_freq = model_cpu.rotary_pos_emb.inv_freq.detach().clone()  # keeps its dtype: bf16 towers build a bf16 table
+    out = vit_oracle.tower_forward(pixels.float(), grid, params, _oracle_cfg(kw), inv_freq=inv_freq)
+    out.backward(gout.float())
+    return out.detach(), {k: p.grad for k, p in params.items()}
+
+
+def _run_gpu(model, pixels, grid, gout):
+    model.to(DEV).train()
+    model.zero_grad(set_to_none=True)
+    out = model(hidden_states=pixels.to(DEV), grid_thw=grid.to(DEV))
+    out.backward(gout.to(device=DEV, dtype=out.dtype))
+    return out.detach(), {n: p.grad.detach() for n, p in model.named_parameters()}
+
+
+CFG1 = dict(depth=4, hidden_size=1280, intermediate_size=3420, num_heads=16, out_hidden_size=2048, fullatt_block_indexes=[3])
+
+
+def test_config1_fp32_parity():
+    """BASELINE config 1: reduced tower, fp32, 2 images of 224x224; outputs and all gradients within 1e-4."""
+    print("[case] config-1 fp32 tower", flush=True)
+    model = _build(CFG1, 0, torch.float32)
+    g = torch.Generator().manual_seed(0)
+    grid = torch.tensor([[1, 16, 16], [1, 16, 16]])
+    pixels = torch.randn(512, 1176, generator=g)
+    gout = torch.randn(128, 2048, generator=g)
+    ref_out, ref_grads = _oracle_run(copy.deepcopy(model), CFG1, pixels, grid, gout)
+    out, grads = _run_gpu(model, pixels, grid, gout)
+    assert out.shape == (128, 2048) and out.dtype == torch.float32
+    assert max_rel_err(out, ref_out) < 1e-4
+    worst = max((max_rel_err(grads[k], ref_grads[k]), k) for k in ref_grads)
+    assert worst[0] < 1e-4, worst
+    assert set(grads) == set(ref_grads)
+
+
+@pytest.mark.parametrize("checkpoint", [False, True])
+def test_small_ragged_tower_bf16_parity(checkpoint):
+    """Ragged images + a video, windows with edge remainders, bf16 kernels vs the fp32 oracle on the same bf16 weights."""
+    print(f"[case] bf16 ragged tower checkpoint={checkpoint}", flush=True)
+    kw = dict(depth=3, hidden_size=1280, intermediate_size=3420, num_heads=16, out_hidden_size=512, fullatt_block_indexes=[1])
+    model = _build(kw, 1, torch.bfloat16)
+    if checkpoint:
+        model.gradient_checkpointing_enable()
+    g = torch.Generator().manual_seed(1)
+    grid = torch.tensor([[1, 18, 22], [2, 8, 12], [1, 34, 16]])
+    S = int((grid[:, 0] * grid[:, 1] * grid[:, 2]).sum())
+    pixels = torch.randn(S, 1176, generator=g).to(torch.bfloat16)
+    gout = torch.randn(S // 4, 512, generator=g).to(torch.bfloat16)
+    ref_out, ref_grads = _oracle_run(copy.deepcopy(model), kw, pixels, grid, gout)
+    out, grads = _run_gpu(model, pixels, grid, gout)
+    assert out.dtype == torch.bfloat16
+    assert max_rel_err(out, ref_out) < 2e-2
+    worst = max((max_rel_err(grads[k], ref_grads[k]), k) for k in ref_grads)
+    assert worst[0] < 2e-2, worst
+
+
+def test_checkpointing_gives_identical_gradients():
+    kw = dict(depth=2, hidden_size=256, intermediate_size=300, num_heads=8, out_hidden_size=256, window_size=56, fullatt_block_indexes=[1])
+    g = torch.Generator().manual_seed(3)
+    grid = torch.tensor([[1, 16, 16], [1, 16, 32]])
+    pixels = torch.randn(768, 1176, generator=g)
+    gout = torch.randn(192, 256, generator=g)
+    res = []
+    for ck in (False, True):
+        model = _build(kw, 5, torch.float32)
+        if ck:
+            model.gradient_checkpointing_enable()
+        res.append(_run_gpu(model, pixels, grid, gout))
+    assert torch.equal(res[0][0], res[1][0])
+    for k in res[0][1]:
+        assert torch.equal(res[0][1][k], res[1][1][k]), k
+
+
+def test_reference_smoke_shape():
+    """The reference's own smoke case (tests/test_ragged_sp_smoke.py:27-98): output [192, 256]."""
+    kw = dict(hidden_size=256, num_heads=8, depth=2, patch_size=14, in_channels=3, out_hidden_size=256, spatial_merge_size=2,
+              window_size=28, fullatt_block_indexes=[1])
+    model = _build(kw, 0, torch.float32).to(DEV).eval()
+    grid = torch.tensor([[1, 16, 16], [1, 16, 32]], dtype=torch.int64)
+    pixels = torch.randn(768, 1176)
+    with torch.no_grad():
+        out = model(pixels.to(DEV), grid.to(DEV))
+    assert out.shape == (192, 256)
+    params = {k: v.detach().float().cpu() for k, v in model.state_dict().items()}
+    ref = vit_oracle.tower_forward(pixels, grid, params, _oracle_cfg(kw))
+    assert ref.shape == (192, 256)
+    assert max_rel_err(out, ref) < 1e-4
+    flat = model(pixels.flatten().to(DEV), grid.to(DEV))  # the reference's GPU tests pass a flat tensor
+    assert torch.equal(flat.detach(), out)
+
+
+def _trainer_config(**over):
+    cfg = dict(seed=0, model_name="unit-test", parallelism="none", dtype="bfloat16", attention_backend="flash_attention_2",
+               activation_checkpointing=False, autocast=True, learning_rate=1e-2, weight_decay=0.01, warmup_ratio=0.0,
+               warmup_steps=0, lr_scheduler_type="cosine", num_iterations=10, max_grad_norm=1.0, profile_time=True,
+               vision_config=dict(depth=2, hidden_size=256, intermediate_size=300, num_heads=8, out_hidden_size=128, fullatt_block_indexes=[1]),
+               synthetic_grids=[[1, 16, 16], [1, 8, 24]])
+    cfg.update(over)
+    return cfg
+
+
+def test_trainer_steps_on_gpu():
+    from mi355_vit.trainer import VisionTrainer
+
+    tr = VisionTrainer(_trainer_config(), rank=0)
+    tr.build_model()
+    tr.initialize_trainer()
+    tr.zero_grad()
+    res = tr.forward_step(iteration=3)
+    emb = res["vision_embeddings"]
+    M = (16 * 16 + 8 * 24) // 4
+    assert emb.shape == (1, M, 128) and emb.dtype == torch.bfloat16 and res["iteration"] == 3 and res["sample_index"] == 0
+    assert res["forward_time_ms"] > 0
+    before = {n: p.detach().clone() for n, p in tr.model.named_parameters()}
+    back = tr.backward_step({"grad": torch.randn(M, 128, device=DEV, dtype=torch.bfloat16)})  # 2-D grad for a 3-D output
+    assert back["backward_time_ms"] > 0
+    contrib = tr.compute_grad_norm_contribution()
+    assert contrib["type"] == "none" and contrib["norm_sq"] > 0
+    coeff = tr.optimizer_step(global_grad_norm=contrib["norm_sq"] ** 0.5)
+    assert coeff == pytest.approx(min(1.0, 1.0 / (contrib["norm_sq"] ** 0.5 + 1e-6)))
+    changed = sum(int(not torch.equal(before[n], p.detach())) for n, p in tr.model.named_parameters())
+    assert changed == len(before)
+    # packed weights follow the optimizer step: a second forward differs from the first
+    res2 = tr.forward_step(iteration=4)
+    assert res2["sample_index"] == 1
+    tr.backward_step(torch.zeros(1, M, 128, device=DEV, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="No pending vision outputs"):
+        tr.backward_step(torch.zeros(1, M, 128, device=DEV))
+    tr.forward_step()
+    with pytest.raises(ValueError, match="No gradient provided"):
+        tr.backward_step(None)
+    stats = tr.get_memory_stats()
+    assert stats["peak_mb"] >= stats["allocated_mb"] > 0
+
+
+def test_trainer_fifo_and_checkpoint_roundtrip(tmp_path):
+    from mi355_vit.trainer import VisionTrainer
+
+    tr = VisionTrainer(_trainer_config(dtype="float32", activation_checkpointing=True, weight_decay=0.0), rank=0)
+    tr.build_model()
+    tr.initialize_trainer()
+    o1 = tr.forward_step(0)["vision_embeddings"]
+    o2 = tr.forward_step(1)["vision_embeddings"]
+    assert len(tr._pending_outputs) == 2 and tr._pending_outputs[0] is o1
+    tr.backward_step(torch.ones_like(o1))
+    assert len(tr._pending_outputs) == 1 and tr._pending_outputs[0] is o2
+    tr.backward_step(torch.ones_like(o2))
+    path = tr.save_checkpoint(str(tmp_path), epoch=2)
+    assert path.endswith("epoch_2/vision/rank_0.pt")
+    sd = torch.load(path, weights_only=True, map_location="cpu")["model"]
+    assert "blocks.0.attn.q_proj.weight" in sd and "merger.mlp.2.bias" in sd and "rotary_pos_emb.inv_freq" not in sd
+    tr.optimizer_step()
+    assert tr.load_checkpoint(str(tmp_path), epoch=2)
+    for k, v in tr.model.state_dict().items():
+        assert torch.equal(v.cpu(), sd[k]), k
+    assert not tr.load_checkpoint(str(tmp_path), epoch=9)
