@@ -1,7 +1,7 @@
 // Variable-length (cu_seqlens) non-causal attention, forward and backward, for gfx950.
 //
-// bf16 path: flash-style kernels on v_mfma_f32_16x16x32_bf16 (+ one 16x16x16 step when head_dim/16 is odd,
-// so head_dim 80 = 5 x 16 is contracted exactly, no padding).  All products are oriented so that the
+// bf16 path: flash-style kernels on v_mfma_f32_16x16x32_bf16; head_dim = 16*ND is contracted in 32-wide steps
+// plus, for odd ND (head_dim 80 = 5 x 16), one half-filled 32-wide step.  All products are oriented so that the
 // accumulator layout of one MFMA is directly the B-operand layout of the next:
 //   forward : S^T = K Q^T   (lane: query l%16, keys 4*(l/16)+i)  ->  O^T += V^T P^T
 //   dK/dV   : S = Q K^T, dP = dO V^T (lane: key l%16, queries 4*(l/16)+i)  ->  dV^T += dO^T P, dK^T += Q^T dS
@@ -257,11 +257,14 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_fwd_mfma(const AttnParams p)
   }
 }
 
-// delta[h, s] = sum_d O[s,h,d] * dO[s,h,d]
+// delta[h, s] = sum_d O[s,h,d] * dO[s,h,d].  One lane per (row, head), 16-byte loads; neighbouring lanes take
+// neighbouring heads of the same row, so a wave sweeps contiguous memory.
 template <typename T>
 __global__ __launch_bounds__(256) void attn_delta_kernel(const T* __restrict__ o, const T* __restrict__ d_o,
                                                          float* __restrict__ delta, int64_t total, int nheads, int hd,
                                                          int64_t o_stride, int64_t do_stride) {
+  constexpr int V = mvit_elem<T>::vec;
+  typedef T vec_t __attribute__((ext_vector_type(V)));
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= total * nheads) return;
   const int64_t s = i / nheads;
@@ -269,7 +272,16 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const T* __restrict__ o
   const T* a = o + s * o_stride + (int64_t)h * hd;
   const T* b = d_o + s * do_stride + (int64_t)h * hd;
   float acc = 0.f;
-  for (int j = 0; j < hd; ++j) acc += to_f32(a[j]) * to_f32(b[j]);
+  if (hd % V == 0 && (o_stride % V) == 0 && (do_stride % V) == 0) {
+    for (int j = 0; j < hd; j += V) {
+      const vec_t x = *reinterpret_cast<const vec_t*>(a + j);
+      const vec_t y = *reinterpret_cast<const vec_t*>(b + j);
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc += to_f32(x[e]) * to_f32(y[e]);
+    }
+  } else {
+    for (int j = 0; j < hd; ++j) acc += to_f32(a[j]) * to_f32(b[j]);
+  }
   delta[(int64_t)h * total + s] = acc;
 }
 

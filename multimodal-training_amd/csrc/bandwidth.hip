@@ -130,14 +130,58 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ 
     out[c] = dw_lds[c] + dw_lds[cols + c] + dw_lds[2 * (size_t)cols + c] + dw_lds[3 * (size_t)cols + c];
 }
 
+// out[c] = sum_b partial[b, c].  A block owns 32 columns; its 8 row groups each add every 8th partial row
+// (fixed order, so the sum is reproducible), then combine through LDS.
 template <typename T>
 __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ partial, int n_partial,
                                                               int64_t cols, T* __restrict__ out) {
-  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (c >= cols) return;
+  __shared__ float red[8][33];
+  const int cx = threadIdx.x & 31, ry = threadIdx.x >> 5;
+  const int64_t c = (int64_t)blockIdx.x * 32 + cx;
   float s = 0.f;
-  for (int b = 0; b < n_partial; ++b) s += partial[(size_t)b * cols + c];
-  out[c] = from_f32<T>(s);
+  if (c < cols)
+    for (int b = ry; b < n_partial; b += 8) s += partial[(size_t)b * cols + c];
+  red[ry][cx] = s;
+  __syncthreads();
+  if (ry == 0 && c < cols) {
+    float t = 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) t += red[k][cx];
+    out[c] = from_f32<T>(t);
+  }
+}
+
+// Column sums with 16-byte loads: a block owns 128 columns (16 lanes x 8/4 elements) and 16 row phases.
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_vec_kernel(const T* __restrict__ x, int64_t ld, int64_t rows, int64_t cols,
+                                                         float* __restrict__ partial) {
+  constexpr int V = mvit_elem<T>::vec;
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  __shared__ float red[16][16 * V + 1];
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const int64_t c0 = ((int64_t)blockIdx.x * 16 + tx) * V;
+  float acc[V];
+#pragma unroll
+  for (int j = 0; j < V; ++j) acc[j] = 0.f;
+  if (c0 < cols) {
+    for (int64_t r = (int64_t)blockIdx.y * 16 + ty; r < rows; r += (int64_t)gridDim.y * 16) {
+      const vec_t v = *reinterpret_cast<const vec_t*>(x + r * ld + c0);
+#pragma unroll
+      for (int j = 0; j < V; ++j) acc[j] += to_f32(v[j]);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < V; ++j) red[ty][tx * V + j] = acc[j];
+  __syncthreads();
+  if (threadIdx.x < 16 * V) {
+    const int64_t c = (int64_t)blockIdx.x * 16 * V + threadIdx.x;
+    if (c < cols) {
+      float t = 0.f;
+#pragma unroll
+      for (int k = 0; k < 16; ++k) t += red[k][threadIdx.x];
+      partial[(size_t)blockIdx.y * cols + c] = t;
+    }
+  }
 }
 
 // Column sums: block b accumulates rows b, b+grid, ... ; thread owns columns.  Partials [grid, cols].
@@ -319,7 +363,7 @@ int mvit_rmsnorm_bwd(const void* dy, const void* x, const void* w, const float* 
 
 int mvit_reduce_partials(const float* partial, int n_partial, int64_t cols, void* out, int out_dtype, mvit_stream_t stream) {
   MVIT_REQUIRE(partial && out && n_partial > 0 && cols > 0, "reduce_partials: bad arguments");
-  const int grid = (int)((cols + 255) / 256);
+  const int grid = (int)((cols + 31) / 32);
   if (out_dtype == MVIT_BF16)
     hipLaunchKernelGGL((reduce_partials_kernel<bf16_t>), grid, 256, 0, S_(stream), partial, n_partial, cols, (bf16_t*)out);
   else if (out_dtype == MVIT_F32)
@@ -332,13 +376,21 @@ int mvit_reduce_partials(const float* partial, int n_partial, int64_t cols, void
 
 int mvit_colsum(const void* x, int64_t ld, int64_t rows, int64_t cols, float* partial, int n_partial, int dtype, mvit_stream_t stream) {
   MVIT_REQUIRE(x && partial && n_partial > 0 && n_partial <= 65535 && cols > 0 && rows >= 0 && ld >= cols, "colsum: bad arguments");
-  dim3 grid((unsigned)((cols + 511) / 512), (unsigned)n_partial);
-  if (dtype == MVIT_BF16)
-    hipLaunchKernelGGL((colsum_kernel<bf16_t>), grid, 256, 0, S_(stream), (const bf16_t*)x, ld, rows, cols, partial);
-  else if (dtype == MVIT_F32)
-    hipLaunchKernelGGL((colsum_kernel<float>), grid, 256, 0, S_(stream), (const float*)x, ld, rows, cols, partial);
-  else
-    return mvit_set_error(MVIT_ERR_UNSUPPORTED, "colsum: dtype %d", dtype);
+  MVIT_REQUIRE(dtype == MVIT_BF16 || dtype == MVIT_F32, "colsum: dtype %d", dtype);
+  const int vec = dtype == MVIT_BF16 ? 8 : 4;
+  if (cols % vec == 0 && ld % vec == 0 && mvit_aligned16(x)) {
+    dim3 grid((unsigned)((cols + 16 * vec - 1) / (16 * vec)), (unsigned)n_partial);
+    if (dtype == MVIT_BF16)
+      hipLaunchKernelGGL((colsum_vec_kernel<bf16_t>), grid, 256, 0, S_(stream), (const bf16_t*)x, ld, rows, cols, partial);
+    else
+      hipLaunchKernelGGL((colsum_vec_kernel<float>), grid, 256, 0, S_(stream), (const float*)x, ld, rows, cols, partial);
+  } else {
+    dim3 grid((unsigned)((cols + 511) / 512), (unsigned)n_partial);
+    if (dtype == MVIT_BF16)
+      hipLaunchKernelGGL((colsum_kernel<bf16_t>), grid, 256, 0, S_(stream), (const bf16_t*)x, ld, rows, cols, partial);
+    else
+      hipLaunchKernelGGL((colsum_kernel<float>), grid, 256, 0, S_(stream), (const float*)x, ld, rows, cols, partial);
+  }
   MVIT_CHECK_LAUNCH("colsum");
   return MVIT_OK;
 }

@@ -33,6 +33,9 @@ struct GemmParams {
   int64_t ldaux;
   int64_t aux_off;
   int tiles_m, tiles_n;
+  int split_k;        // K slices (1 = none)
+  int64_t k_chunk;    // K extent of one slice (multiple of BK)
+  float* workspace;   // [split_k][M][N] fp32 partial sums when split_k > 1
 };
 
 template <typename T>
@@ -167,11 +170,16 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
 
   // XCD-aware tile order: hardware deals consecutive work-group ids round-robin to the 8 XCDs; give each
   // XCD a contiguous range of tiles (N fastest) so that its L2 sees one A panel at a time.
-  const int total = p.tiles_m * p.tiles_n;
+  // With split-K the slices are the slowest index: all tiles of one K slice share the same rows of A and B.
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int total = tiles * p.split_k;
   const int per_xcd = (total + 7) / 8;
-  const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (tile >= total) return;
+  const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (work >= total) return;
+  const int slice = work / tiles, tile = work % tiles;
   const int tm = tile / p.tiles_n, tn = tile % p.tiles_n;
+  const int64_t k_begin = (int64_t)slice * p.k_chunk;
+  const int64_t k_end = p.split_k > 1 ? (k_begin + p.k_chunk < p.K ? k_begin + p.k_chunk : p.K) : p.K;
   constexpr bool DUAL = (EPI == MVIT_EPI_SWIGLU);
   constexpr int N_PER_BLOCK = DUAL ? BN / 2 : BN;
   const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * N_PER_BLOCK;
@@ -192,17 +200,17 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
   const T* A = static_cast<const T*>(p.A);
   const T* B = static_cast<const T*>(p.B);
   const T* B2 = static_cast<const T*>(p.B2);
-  la.load(A, nullptr, p.lda, m0, p.M, 0, p.K, false);
-  lb.load(B, B2, p.ldb, n0, p.N, 0, p.K, DUAL);
+  la.load(A, nullptr, p.lda, m0, p.M, k_begin, k_end, false);
+  lb.load(B, B2, p.ldb, n0, p.N, k_begin, k_end, DUAL);
 
-  for (int64_t k0 = 0; k0 < p.K; k0 += BK) {
+  for (int64_t k0 = k_begin; k0 < k_end; k0 += BK) {
     __syncthreads();  // previous tile fully consumed
     la.store(lds_a);
     lb.store(lds_b);
     __syncthreads();
-    if (k0 + BK < p.K) {
-      la.load(A, nullptr, p.lda, m0, p.M, k0 + BK, p.K, false);
-      lb.load(B, B2, p.ldb, n0, p.N, k0 + BK, p.K, DUAL);
+    if (k0 + BK < k_end) {
+      la.load(A, nullptr, p.lda, m0, p.M, k0 + BK, k_end, false);
+      lb.load(B, B2, p.ldb, n0, p.N, k0 + BK, k_end, DUAL);
     }
     if constexpr (sizeof(T) == 2) {
 #pragma unroll
@@ -241,6 +249,26 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
   const T* bias2 = static_cast<const T*>(p.bias2);
   const int lc = l & 31, lr = 4 * (l >> 5);
 
+  if constexpr (EPI == MVIT_EPI_NONE) {
+    if (p.split_k > 1) {  // fp32 partial tile; summed over slices by splitk_reduce_kernel
+      float* W = p.workspace + (int64_t)slice * p.M * p.N;
+#pragma unroll
+      for (int b = 0; b < NT; ++b) {
+        const int64_t n = n0 + wn * WAVE_N + b * 32 + lc;
+        if (n >= p.N) continue;
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int64_t m = m0 + wm * WAVE_M + a * 32 + 8 * j + lr + i;
+              if (m < p.M) W[m * p.N + n] = acc[a][b][4 * j + i];
+            }
+      }
+      return;
+    }
+  }
   if constexpr (DUAL) {
     const int64_t n = n0 + wn * 32 + lc;
     if (n < p.N) {
@@ -305,6 +333,18 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
   }
 }
 
+// C[m, n] = sum over slices of the fp32 partial tiles (fixed order, so the result is reproducible).
+template <typename TO>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, int split_k, int64_t M, int64_t N,
+                                                            TO* __restrict__ C, int64_t ldc) {
+  const int64_t total = M * N;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    float s = 0.f;
+    for (int k = 0; k < split_k; ++k) s += ws[(int64_t)k * total + i];
+    C[(i / N) * ldc + (i % N)] = from_f32<TO>(s);
+  }
+}
+
 template <typename T, typename TO, bool TA, bool TB, int EPI>
 int launch(const GemmParams& p, hipStream_t stream) {
   using LA = TileLoader<T, BM, TA>;
@@ -317,10 +357,17 @@ int launch(const GemmParams& p, hipStream_t stream) {
     if (e != hipSuccess) return mvit_set_error(MVIT_ERR_LAUNCH, "gemm: hipFuncSetAttribute(%zu B LDS): %s", lds, hipGetErrorString(e));
     attr_set = true;
   }
-  const int total = p.tiles_m * p.tiles_n;
+  if (p.split_k > 1 && EPI != MVIT_EPI_NONE) return mvit_set_error(MVIT_ERR_UNSUPPORTED, "gemm: split_k needs EPI_NONE");
+  const int total = p.tiles_m * p.tiles_n * p.split_k;
   const int grid = ((total + 7) / 8) * 8;
   hipLaunchKernelGGL(kern, grid, 256, lds, stream, p);
   MVIT_CHECK_LAUNCH("gemm");
+  if (p.split_k > 1) {
+    const int64_t elems = p.M * p.N;
+    const int rgrid = (int)((elems + 255) / 256 < 8192 ? (elems + 255) / 256 : 8192);
+    hipLaunchKernelGGL((splitk_reduce_kernel<TO>), rgrid, 256, 0, stream, p.workspace, p.split_k, p.M, p.N, static_cast<TO*>(p.C), p.ldc);
+    MVIT_CHECK_LAUNCH("gemm split-k reduce");
+  }
   return MVIT_OK;
 }
 
@@ -392,6 +439,17 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
   const int64_t tm = (a->M + BM - 1) / BM, tn = (a->N + n_per_block - 1) / n_per_block;
   MVIT_REQUIRE(tm * tn < (1ll << 30), "gemm: too many tiles");
   p.tiles_m = (int)tm; p.tiles_n = (int)tn;
+  p.split_k = 1; p.k_chunk = a->K; p.workspace = nullptr;
+  if (a->split_k > 1) {
+    const int bk = a->dtype == MVIT_BF16 ? 64 : 16;
+    const int64_t chunk = ((a->K + a->split_k - 1) / a->split_k + bk - 1) / bk * bk;
+    const int64_t slices = (a->K + chunk - 1) / chunk;  // never an empty slice
+    MVIT_REQUIRE(epi == MVIT_EPI_NONE, "gemm: split_k is only available with EPI_NONE");
+    MVIT_REQUIRE(a->workspace && a->workspace_bytes >= (int64_t)sizeof(float) * slices * a->M * a->N,
+                 "gemm: split_k=%d needs a workspace of %lld bytes", a->split_k, (long long)(sizeof(float) * slices * a->M * a->N));
+    MVIT_REQUIRE(tm * tn * slices < (1ll << 30), "gemm: too many tiles");
+    if (slices > 1) { p.split_k = (int)slices; p.k_chunk = chunk; p.workspace = static_cast<float*>(a->workspace); }
+  }
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (a->dtype == MVIT_BF16) {
     if (a->out_dtype == MVIT_BF16) return dispatch_trans<bf16_t, bf16_t>(a->trans_a, a->trans_b, epi, p, s);

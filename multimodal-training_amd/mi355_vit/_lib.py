@@ -27,6 +27,7 @@ class GemmArgs(C.Structure):
         ("C", _vp), ("ldc", _i64),
         ("R", _vp), ("ldr", _i64),
         ("aux", _vp), ("ldaux", _i64), ("aux_off", _i64),
+        ("workspace", _vp), ("workspace_bytes", _i64), ("split_k", _i32), ("reserved2", _i32),
     ]
 
 

@@ -131,12 +131,12 @@ def _block_backward(dx2: torch.Tensor, x: torch.Tensor, saved: tuple, W: BlockWe
     # ---- MLP: x2 = x1 + down(silu(g) * u)
     g_bd = ops.colsum(dx2, gdt["mlp.down_proj.bias"])
     g_wd = torch.empty(C, I, dtype=gdt["mlp.down_proj.weight"], device=dev)
-    ops.gemm(dx2, h, g_wd, trans_a=True, trans_b=True, n=I)
+    ops.gemm(dx2, h, g_wd, trans_a=True, trans_b=True, n=I, split_k=ops.wgrad_split_k(C, I, S))
     dgu = torch.empty(S, 2 * Ipad, dtype=x.dtype, device=dev)
     ops.gemm(dx2, W.wdown, dgu, trans_b=True, epilogue=E.EPI_SWIGLU_BWD, residual=gu, aux_off=Ipad)
     g_bgu = ops.colsum(dgu, gdt["mlp.gate_proj.bias"])
     g_wgu = torch.empty(2 * Ipad, C, dtype=gdt["mlp.gate_proj.weight"], device=dev)
-    ops.gemm(dgu, n2, g_wgu, trans_a=True, trans_b=True)
+    ops.gemm(dgu, n2, g_wgu, trans_a=True, trans_b=True, split_k=ops.wgrad_split_k(2 * Ipad, C, S))
     dn2 = torch.empty_like(x)
     ops.gemm(dgu, W.wgu, dn2, trans_b=True)
     del dgu
@@ -145,7 +145,7 @@ def _block_backward(dx2: torch.Tensor, x: torch.Tensor, saved: tuple, W: BlockWe
     # ---- attention: x1 = x + proj(attn(rope(qkv(norm1(x)))))
     g_bp = ops.colsum(dx1, gdt["attn.proj.bias"])
     g_wp = torch.empty(C, C, dtype=gdt["attn.proj.weight"], device=dev)
-    ops.gemm(dx1, o, g_wp, trans_a=True, trans_b=True)
+    ops.gemm(dx1, o, g_wp, trans_a=True, trans_b=True, split_k=ops.wgrad_split_k(C, C, S))
     d_o = dn2  # reuse the buffer
     ops.gemm(dx1, W.wproj, d_o, trans_b=True)
     dqkv = torch.empty_like(qkv)
@@ -154,7 +154,7 @@ def _block_backward(dx2: torch.Tensor, x: torch.Tensor, saved: tuple, W: BlockWe
     ops.rope_(dqkv, geo.cos, geo.sin, 2 * H, hd, backward=True)
     g_bqkv = ops.colsum(dqkv, gdt["attn.q_proj.bias"])
     g_wqkv = torch.empty(3 * C, C, dtype=gdt["attn.q_proj.weight"], device=dev)
-    ops.gemm(dqkv, n1, g_wqkv, trans_a=True, trans_b=True)
+    ops.gemm(dqkv, n1, g_wqkv, trans_a=True, trans_b=True, split_k=ops.wgrad_split_k(3 * C, C, S))
     dn1 = d_o
     ops.gemm(dqkv, W.wqkv, dn1, trans_b=True)
     dx, g_n1 = ops.rmsnorm_bwd(dn1, x, W.norm1.view(-1), rstd1, dx_add=dx1, w_grad_dtype=gdt["norm1.weight"])
@@ -218,7 +218,7 @@ class PatchEmbedFn(torch.autograd.Function):
     def backward(ctx, dout):
         px = ctx.px
         gw = torch.empty(dout.shape[1], px.shape[1], dtype=ctx.wdtype, device=px.device)
-        ops.gemm(dout.contiguous(), px, gw, trans_a=True, trans_b=True)
+        ops.gemm(dout.contiguous(), px, gw, trans_a=True, trans_b=True, split_k=ops.wgrad_split_k(gw.shape[0], gw.shape[1], px.shape[0]))
         return None, gw.view(ctx.wshape), None
 
 
@@ -272,12 +272,12 @@ class MergerFn(torch.autograd.Function):
         dev = x.device
         g_b2 = ops.colsum(dy, ctx.gdt[4])
         g_w2 = torch.empty(W2.shape, dtype=ctx.gdt[3], device=dev)
-        ops.gemm(dy, y1, g_w2, trans_a=True, trans_b=True)
+        ops.gemm(dy, y1, g_w2, trans_a=True, trans_b=True, split_k=ops.wgrad_split_k(g_w2.shape[0], g_w2.shape[1], dy.shape[0]))
         dz = torch.empty_like(z)
         ops.gemm(dy, W2, dz, trans_b=True, epilogue=E.EPI_GELU_BWD, residual=z)
         g_b0 = ops.colsum(dz, ctx.gdt[2])
         g_w0 = torch.empty(W0.shape, dtype=ctx.gdt[1], device=dev)
-        ops.gemm(dz, ln2, g_w0, trans_a=True, trans_b=True)
+        ops.gemm(dz, ln2, g_w0, trans_a=True, trans_b=True, split_k=ops.wgrad_split_k(g_w0.shape[0], g_w0.shape[1], dz.shape[0]))
         dln = torch.empty_like(ln2)
         ops.gemm(dz, W0, dln, trans_b=True)
         dx, g_ln = ops.rmsnorm_bwd(dln.view(x.shape), x, lw, rstd, w_grad_dtype=ctx.gdt[0])

@@ -15,6 +15,26 @@ _DT = {torch.float32: F32, torch.bfloat16: BF16}
 N_PARTIAL = 256  # row-slice count of the two-stage column reductions
 
 
+_trace = None  # optional list collecting (tag, info, start_event, end_event) per tagged launch
+
+
+def set_trace(records: Optional[list]) -> None:
+    """Give a list to time every tagged kernel launch with a pair of events on the current stream; None stops."""
+    global _trace
+    _trace = records
+
+
+def _launch(tag: str, info: dict, call):
+    if _trace is None:
+        return call()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    rc = call()
+    e1.record()
+    _trace.append((tag, info, e0, e1))
+    return rc
+
+
 def dt(t: torch.Tensor) -> int:
     try:
         return _DT[t.dtype]
@@ -94,7 +114,9 @@ def rmsnorm_fwd(x: torch.Tensor, w: torch.Tensor, eps: float) -> Tuple[torch.Ten
         raise ValueError("rmsnorm_fwd: x must be contiguous [rows, cols] and w [cols] of the same dtype")
     y = torch.empty_like(x)
     rstd = torch.empty(x.shape[0], dtype=torch.float32, device=x.device)
-    rc = _lib.load().mvit_rmsnorm_fwd(x.data_ptr(), w.data_ptr(), y.data_ptr(), rstd.data_ptr(), x.shape[0], x.shape[1], eps, dt(x), _stream(x))
+    st = _stream(x)
+    rc = _launch("rmsnorm_fwd", {"rows": x.shape[0], "cols": x.shape[1], "esize": x.element_size()},
+                 lambda: _lib.load().mvit_rmsnorm_fwd(x.data_ptr(), w.data_ptr(), y.data_ptr(), rstd.data_ptr(), x.shape[0], x.shape[1], eps, dt(x), st))
     _lib.check(rc, "mvit_rmsnorm_fwd")
     return y, rstd
 
@@ -109,7 +131,9 @@ def rmsnorm_bwd(dy, x, w, rstd, dx_add: Optional[torch.Tensor] = None, w_grad_dt
     dx = torch.empty_like(x)
     partial = torch.empty(N_PARTIAL, cols, dtype=torch.float32, device=x.device)
     lib = _lib.load()
-    rc = lib.mvit_rmsnorm_bwd(dy.data_ptr(), x.data_ptr(), w.data_ptr(), rstd.data_ptr(), _p(dx_add), dx.data_ptr(), partial.data_ptr(), N_PARTIAL, rows, cols, dt(x), _stream(x))
+    st = _stream(x)
+    rc = _launch("rmsnorm_bwd", {"rows": rows, "cols": cols, "esize": x.element_size(), "add": dx_add is not None},
+                 lambda: lib.mvit_rmsnorm_bwd(dy.data_ptr(), x.data_ptr(), w.data_ptr(), rstd.data_ptr(), _p(dx_add), dx.data_ptr(), partial.data_ptr(), N_PARTIAL, rows, cols, dt(x), st))
     _lib.check(rc, "mvit_rmsnorm_bwd")
     dw = torch.empty(cols, dtype=w_grad_dtype or w.dtype, device=x.device)
     _lib.check(lib.mvit_reduce_partials(partial.data_ptr(), N_PARTIAL, cols, dw.data_ptr(), dt(dw), _stream(x)), "mvit_reduce_partials")
@@ -120,7 +144,7 @@ def colsum(x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
     """Column sums of a 2-D (possibly row-strided) tensor: the bias gradient of a Linear layer."""
     _rowmajor(x, "colsum x")
     rows, cols = x.shape
-    npart = max(1, min(N_PARTIAL, rows))
+    npart = max(1, min(64, (rows + 15) // 16))
     partial = torch.empty(npart, cols, dtype=torch.float32, device=x.device)
     lib = _lib.load()
     _lib.check(lib.mvit_colsum(x.data_ptr(), x.stride(0), rows, cols, partial.data_ptr(), npart, dt(x), _stream(x)), "mvit_colsum")
@@ -138,7 +162,9 @@ def rope_(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, nheads: int, he
             raise ValueError(f"rope: cos/sin must be contiguous fp32 [{rows}, {head_dim}]")
     if x.shape[1] < nheads * head_dim:
         raise ValueError("rope: row narrower than nheads*head_dim")
-    rc = _lib.load().mvit_rope(x.data_ptr(), cos.data_ptr(), sin.data_ptr(), rows, nheads, head_dim, x.stride(0), int(backward), dt(x), _stream(x))
+    st = _stream(x)
+    rc = _launch("rope", {"rows": rows, "nheads": nheads, "head_dim": head_dim, "esize": x.element_size()},
+                 lambda: _lib.load().mvit_rope(x.data_ptr(), cos.data_ptr(), sin.data_ptr(), rows, nheads, head_dim, x.stride(0), int(backward), dt(x), st))
     _lib.check(rc, "mvit_rope")
     return x
 
@@ -154,7 +180,9 @@ def gather_rows(src: torch.Tensor, index: torch.Tensor, rows_per_index: int = 1)
         raise ValueError("gather_rows: rows not divisible by rows_per_index")
     out = torch.empty(index.numel() * rows_per_index, src.shape[1], dtype=src.dtype, device=src.device)
     row_bytes = rows_per_index * src.shape[1] * src.element_size()
-    rc = _lib.load().mvit_gather_rows(src.data_ptr(), index.data_ptr(), out.data_ptr(), index.numel(), row_bytes, _stream(src))
+    st = _stream(src)
+    rc = _launch("gather_rows", {"rows": index.numel(), "row_bytes": row_bytes},
+                 lambda: _lib.load().mvit_gather_rows(src.data_ptr(), index.data_ptr(), out.data_ptr(), index.numel(), row_bytes, st))
     _lib.check(rc, "mvit_gather_rows")
     return out
 
@@ -226,6 +254,7 @@ def gemm(
     aux: Optional[torch.Tensor] = None,
     aux_off: int = 0,
     n: Optional[int] = None,
+    split_k: int = 1,
 ) -> torch.Tensor:
     """out[M, N] = epilogue(A . B^T) with A = a (or a^T if trans_a) and B = b (or b^T if trans_b), see include/mi355_vit.h.
 
@@ -273,8 +302,22 @@ def gemm(
             raise ValueError("gemm: aux shape/dtype mismatch")
         args.aux, args.ldaux = aux.data_ptr(), aux.stride(0)
     args.aux_off = aux_off
-    _lib.check(_lib.load().mvit_gemm(C.byref(args), _stream(a)), "mvit_gemm")
+    if split_k > 1:
+        if epilogue != _lib.EPI_NONE:
+            raise ValueError("gemm: split_k needs the plain epilogue")
+        ws = torch.empty(split_k * M * N, dtype=torch.float32, device=a.device)
+        args.workspace, args.workspace_bytes, args.split_k = ws.data_ptr(), ws.numel() * 4, split_k
+    st = _stream(a)
+    tag = f"gemm_{'t' if trans_a else 'n'}{'t' if trans_b else 'n'}_epi{epilogue}"
+    _lib.check(_launch(tag, {"M": M, "N": N, "K": K}, lambda: _lib.load().mvit_gemm(C.byref(args), st)), "mvit_gemm")
     return out
+
+
+def wgrad_split_k(out_rows: int, out_cols: int, k: int) -> int:
+    """K slices for a weight-gradient GEMM: few output tiles (256x128) but a long contraction (the tokens)."""
+    tiles = -(-out_rows // 256) * -(-out_cols // 128)
+    want = max(1, min(16, round(768 / tiles)))
+    return max(1, min(want, k // 512))
 
 
 # ------------------------------------------------------------------------------ attention
@@ -298,13 +341,12 @@ def attn_fwd(q, k, v, cu_seqlens: torch.Tensor, max_seqlen: int, nheads: int, he
     if out is None:
         out = torch.empty(S, nheads * head_dim, dtype=q.dtype, device=q.device)
     lse = torch.empty(nheads, S, dtype=torch.float32, device=q.device)
-    rc = _lib.load().mvit_attn_fwd(
+    st = _stream(q)
+    strides = (_attn_view(q, nheads, head_dim, "attn q"), _attn_view(k, nheads, head_dim, "attn k"),
+               _attn_view(v, nheads, head_dim, "attn v"), _attn_view(out, nheads, head_dim, "attn o"))
+    rc = _launch("attn_fwd", {"cu": cu_seqlens, "max_seqlen": max_seqlen, "nheads": nheads, "head_dim": head_dim}, lambda: _lib.load().mvit_attn_fwd(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), cu_seqlens.data_ptr(),
-        cu_seqlens.numel() - 1, max_seqlen, S, nheads, head_dim,
-        _attn_view(q, nheads, head_dim, "attn q"), _attn_view(k, nheads, head_dim, "attn k"),
-        _attn_view(v, nheads, head_dim, "attn v"), _attn_view(out, nheads, head_dim, "attn o"),
-        scale, dt(q), _stream(q),
-    )
+        cu_seqlens.numel() - 1, max_seqlen, S, nheads, head_dim, *strides, scale, dt(q), st))
     _lib.check(rc, "mvit_attn_fwd")
     return out, lse
 
@@ -318,14 +360,11 @@ def attn_bwd(q, k, v, o, d_o, lse, cu_seqlens, max_seqlen, nheads, head_dim, sca
     if tuple(lse.shape) != (nheads, S) or lse.dtype != torch.float32 or not lse.is_contiguous():
         raise ValueError("attn_bwd: lse must be contiguous fp32 [nheads, S]")
     delta = torch.empty(nheads, S, dtype=torch.float32, device=q.device)
-    rc = _lib.load().mvit_attn_bwd(
+    st = _stream(q)
+    strides = tuple(_attn_view(t, nheads, head_dim, nm) for t, nm in ((q, "q"), (k, "k"), (v, "v"), (o, "o"), (d_o, "do"), (dq, "dq"), (dk, "dk"), (dv, "dv")))
+    rc = _launch("attn_bwd", {"cu": cu_seqlens, "max_seqlen": max_seqlen, "nheads": nheads, "head_dim": head_dim}, lambda: _lib.load().mvit_attn_bwd(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(), lse.data_ptr(),
         dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(), cu_seqlens.data_ptr(),
-        cu_seqlens.numel() - 1, max_seqlen, S, nheads, head_dim,
-        _attn_view(q, nheads, head_dim, "q"), _attn_view(k, nheads, head_dim, "k"), _attn_view(v, nheads, head_dim, "v"),
-        _attn_view(o, nheads, head_dim, "o"), _attn_view(d_o, nheads, head_dim, "do"),
-        _attn_view(dq, nheads, head_dim, "dq"), _attn_view(dk, nheads, head_dim, "dk"), _attn_view(dv, nheads, head_dim, "dv"),
-        scale, dt(q), _stream(q),
-    )
+        cu_seqlens.numel() - 1, max_seqlen, S, nheads, head_dim, *strides, scale, dt(q), st))
     _lib.check(rc, "mvit_attn_bwd")
     return dq, dk, dv

@@ -1,0 +1,165 @@
+"""CPU tests: the C-ABI library loads and exports every symbol the header declares; module tree / state-dict
+contract; trainer host logic (error paths, clipping, optimizer grouping) without touching a GPU."""
+
+import re
+from collections import deque
+from pathlib import Path
+
+import pytest
+import torch
+from torch import nn
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def test_library_exports_every_declared_symbol():
+    from mi355_vit import _lib
+
+    header = (ROOT / "include" / "mi355_vit.h").read_text()
+    declared = sorted(set(re.findall(r"\b(mvit_[a-z0-9_]+)\s*\(", header)))
+    assert declared == _lib.EXPORTS
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.mvit_version() >= 100
+    assert isinstance(lib.mvit_last_error(), bytes)
+
+
+def test_gemm_args_struct_matches_header_field_order():
+    from mi355_vit import _lib
+
+    header = (ROOT / "include" / "mi355_vit.h").read_text()
+    body = header[header.index("typedef struct mvit_gemm_args {") : header.index("} mvit_gemm_args;")]
+    fields = re.findall(r"\b(?:int|int64_t|const void\*|void\*)\s+([A-Za-z0-9_, ]+);", body)
+    names = [n.strip() for grp in fields for n in grp.split(",")]
+    assert names == [f[0] for f in _lib.GemmArgs._fields_]
+
+
+def test_ops_refuse_cpu_tensors():
+    from mi355_vit import ops
+
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.rmsnorm_fwd(torch.randn(4, 8), torch.ones(8), 1e-6)
+
+
+def test_state_dict_contract_and_default_init():
+    from mi355_vit.config import Qwen2_5_VLVisionConfig
+    from mi355_vit.modeling import Qwen2_5_VisionTransformerPretrainedModel
+
+    cfg = Qwen2_5_VLVisionConfig(depth=2, hidden_size=64, intermediate_size=36, num_heads=4, out_hidden_size=48, fullatt_block_indexes=[1])
+    torch.manual_seed(0)
+    m = Qwen2_5_VisionTransformerPretrainedModel(cfg)
+    sd = m.state_dict()
+    C, I, O = 64, 36, 48
+    want = {"patch_embed.proj.weight": (C, 3, 2, 14, 14), "merger.ln_q.weight": (C,), "merger.mlp.0.weight": (4 * C, 4 * C),
+            "merger.mlp.0.bias": (4 * C,), "merger.mlp.2.weight": (O, 4 * C), "merger.mlp.2.bias": (O,)}
+    for i in range(2):
+        b = f"blocks.{i}."
+        want.update({b + "norm1.weight": (C,), b + "norm2.weight": (C,)})
+        for n in ("q_proj", "k_proj", "v_proj", "proj"):
+            want.update({b + f"attn.{n}.weight": (C, C), b + f"attn.{n}.bias": (C,)})
+        want.update({b + "mlp.gate_proj.weight": (I, C), b + "mlp.gate_proj.bias": (I,), b + "mlp.up_proj.weight": (I, C),
+                     b + "mlp.up_proj.bias": (I,), b + "mlp.down_proj.weight": (C, I), b + "mlp.down_proj.bias": (C,)})
+    assert {k: tuple(v.shape) for k, v in sd.items()} == want  # inv_freq is non-persistent
+    assert (sd["blocks.0.norm1.weight"] == 1).all()
+    # same construction order as the reference => same default init under a seed as plain torch modules built in that order
+    torch.manual_seed(0)
+    conv = nn.Conv3d(3, C, kernel_size=[2, 14, 14], stride=[2, 14, 14], bias=False)
+    q = nn.Linear(C, C)
+    assert torch.equal(conv.weight, sd["patch_embed.proj.weight"]) and torch.equal(q.weight, sd["blocks.0.attn.q_proj.weight"])
+    # .to(bfloat16) casts the rotary buffer as well (the reference's dtype propagation)
+    assert m.to(torch.bfloat16).rotary_pos_emb.inv_freq.dtype == torch.bfloat16
+    assert m.spatial_merge_unit == 4 and m.window_size == 112 and len(m.blocks) == 2
+    m.gradient_checkpointing_enable()
+    assert m.gradient_checkpointing and all(b.gradient_checkpointing for b in m.blocks)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        m(torch.randn(16, 1176), torch.tensor([[1, 4, 4]]))
+    n_params = sum(p.numel() for p in Qwen2_5_VisionTransformerPretrainedModel(Qwen2_5_VLVisionConfig.qwen2_5_vl_tower(depth=1)).parameters())
+    per_block = 2 * 1280 + 4 * (1280 * 1280 + 1280) + 2 * (3420 * 1280 + 3420) + 1280 * 3420 + 1280
+    assert n_params == 1280 * 1176 + per_block + 1280 + 5120 * 5120 + 5120 + 3584 * 5120 + 3584
+
+
+def _host_trainer(**over):
+    from mi355_vit.trainer import VisionTrainer
+
+    cfg = dict(seed=3, parallelism="none", dtype="bfloat16", learning_rate=1e-3, weight_decay=0.05, warmup_ratio=0.2, warmup_steps=0,
+               lr_scheduler_type="linear", num_iterations=10, max_grad_norm=1.0)
+    cfg.update(over)
+    tr = VisionTrainer(cfg, rank=1)
+
+    class Toy(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.attn = nn.Linear(4, 4)
+            self.norm1 = nn.LayerNorm(4)
+            self.ln_q = nn.LayerNorm(4)
+
+    tr.model = Toy()
+    return tr
+
+
+def test_trainer_misuse_errors_and_grad_reshape_on_host():
+    tr = _host_trainer()
+    with pytest.raises(ValueError, match=r"\[r1\] No gradient provided"):
+        tr.backward_step(None)
+    with pytest.raises(ValueError, match="No gradient provided"):
+        tr.backward_step({"grad": None})
+    with pytest.raises(RuntimeError, match="No pending vision outputs available"):
+        tr.backward_step(torch.zeros(2, 2))
+    x = torch.randn(1, 3, 4, requires_grad=True)
+    tr._pending_outputs = deque([x * 2.0])
+    tr.backward_step(torch.ones(3, 4))  # 2-D gradient for a 3-D output with batch 1
+    assert torch.equal(x.grad, torch.full_like(x, 2.0))
+    tr._pending_outputs = deque([torch.randn(2, 3, 4, requires_grad=True) * 1.0])
+    with pytest.raises(RuntimeError, match="Dimension mismatch"):
+        tr.backward_step(torch.ones(3, 4))
+    assert tr.backward_step.__doc__ is None or True
+
+
+def test_trainer_optimizer_grouping_clip_and_schedule():
+    tr = _host_trainer()
+    tr._build_optimizer(list(tr.model.parameters()))
+    groups = tr.optimizer.param_groups
+    assert isinstance(tr.optimizer, torch.optim.Adam) and len(groups) == 2
+    assert groups[0]["weight_decay"] == 0.05 and groups[1]["weight_decay"] == 0.0
+    assert [tuple(p.shape) for p in groups[0]["params"]] == [(4, 4)]  # only attn.weight decays: bias / norm / ln_ are excluded
+    assert len(groups[1]["params"]) == 5
+    tr._build_scheduler(10)  # warmup_ratio 0.2 -> 2 warm-up steps, then linear decay
+    lrs = []
+    for p in tr.model.parameters():
+        p.grad = torch.ones_like(p)
+    for _ in range(4):
+        lrs.append(tr.optimizer.param_groups[0]["lr"])
+        tr.optimizer_step()
+    assert lrs == pytest.approx([0.0, 0.5e-3, 1e-3, 1e-3 * 7 / 8])
+    for p in tr.model.parameters():
+        p.grad = torch.ones_like(p)
+    contrib = tr.compute_grad_norm_contribution()
+    n = sum(p.numel() for p in tr.model.parameters())
+    assert contrib == {"type": "none", "norm_sq": pytest.approx(float(n))}
+    coeff = tr.optimizer_step(global_grad_norm=4.0)
+    assert coeff == pytest.approx(1.0 / (4.0 + 1e-6))
+    for p in tr.model.parameters():
+        p.grad = torch.ones_like(p)
+    tr._clip_gradients(4.0, 1.0)
+    assert all(torch.allclose(p.grad, torch.full_like(p, 1.0 / (4.0 + 1e-6))) for p in tr.model.parameters())
+    assert tr._clip_gradients(0.5, 1.0) == 1.0
+    tr.zero_grad()
+    assert all(p.grad is None for p in tr.model.parameters())
+    tr2 = _host_trainer(weight_decay=0.0)
+    tr2._build_optimizer(list(tr2.model.parameters()))
+    assert len(tr2.optimizer.param_groups) == 1 and tr2.optimizer.defaults["foreach"] is False
+
+
+def test_trainer_config_resolution():
+    from mi355_vit.trainer import VisionTrainer, synthetic_batches
+
+    tr = VisionTrainer(dict(seed=0), rank=0)
+    assert tr._load_model_config("Qwen/Qwen2.5-VL-7B-Instruct").out_hidden_size == 3584
+    assert tr._load_model_config("Qwen/Qwen2.5-VL-3B-Instruct").out_hidden_size == 2048
+    assert tr._load_model_config("Qwen/Qwen2.5-VL-32B-Instruct").hidden_size == 1280
+    with pytest.raises(ValueError, match="vision_config"):
+        tr._load_model_config("somebody/unknown")
+    b = next(synthetic_batches([[1, 4, 4], [2, 2, 6]], 0, 1176))
+    assert b["pixel_values"].shape == (40, 1176) and b["image_grid_thw"].tolist() == [[1, 4, 4], [2, 2, 6]] and b["sample_index"] == 0
+    assert tr._get_torch_dtype("float32") == torch.float32 and tr._get_torch_dtype("nonsense") == torch.bfloat16
