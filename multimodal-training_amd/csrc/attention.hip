@@ -138,14 +138,58 @@ __device__ __forceinline__ void stage_tile(bf16_t* tile, const bf16_t* src, int6
   }
 }
 
+// The same copy split in two halves (global -> registers, registers -> LDS) with the per-thread chunk
+// coordinates computed once, so that the loads of the next tile can be in flight while the current one is used.
+template <int ND, int ROWS, int PITCH, int NTHREADS>
+struct TileStager {
+  using G = Geo<ND>;
+  static constexpr int CHUNKS = ROWS * G::CH;
+  static constexpr int PER = (CHUNKS + NTHREADS - 1) / NTHREADS;
+  int row[PER];      // tile row of chunk i (ROWS = "no chunk")
+  int lds_off[PER];  // element offset in the LDS tile
+  int64_t goff[PER]; // element offset from the tile's first row in global memory
+  bf16x8 regs[PER];
+
+  __device__ __forceinline__ void init(int64_t stride) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int c = threadIdx.x + NTHREADS * i;
+      const int r = c / G::CH, dc = c % G::CH;
+      row[i] = c < CHUNKS ? r : ROWS;
+      lds_off[i] = r * PITCH + dc * 8;
+      goff[i] = (int64_t)r * stride + dc * 8;
+    }
+  }
+  __device__ __forceinline__ void load(const bf16_t* src, int valid_rows) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      bf16x8 v;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = (bf16_t)0.f;
+      if (row[i] < valid_rows) v = *reinterpret_cast<const bf16x8*>(src + goff[i]);
+      regs[i] = v;
+    }
+  }
+  __device__ __forceinline__ void store(bf16_t* tile) const {
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+      if (row[i] < ROWS) *reinterpret_cast<bf16x8*>(tile + lds_off[i]) = regs[i];
+  }
+};
+
+__device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
+
 // ================================================================================================
 // Forward.  Block = NWAVES waves = 64*NWAVES queries of one (segment, head); 64 keys per iteration.
-template <int ND, int NWAVES>
-__global__ __launch_bounds__(64 * NWAVES) void attn_fwd_mfma(const AttnParams p) {
+// Two work-groups share a CU (<= 256 registers), K/V tiles are double buffered in LDS and the next tile is
+// fetched while the current one is used; key masking only runs on a segment's last, partial tile; the output
+// accumulators are rescaled only in iterations where some row maximum of the wave actually grew.
+template <int ND, int NWAVES, int BNK, bool PIPE>
+__global__ __launch_bounds__(64 * NWAVES, 2) void attn_fwd_mfma(const AttnParams p) {
   using G = Geo<ND>;
-  constexpr int HD = G::HD, BNK = 64, NT = 64 * NWAVES;
-  __shared__ __attribute__((aligned(16))) bf16_t lds_k[BNK * G::PK];
-  __shared__ __attribute__((aligned(16))) bf16_t lds_v[BNK * G::PV];
+  constexpr int HD = G::HD, NT = 64 * NWAVES, KT = BNK / 16, KK = BNK / 32, NBUF = PIPE ? 2 : 1;
+  __shared__ __attribute__((aligned(16))) bf16_t lds_k[NBUF][BNK * G::PK];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_v[NBUF][BNK * G::PV];
 
   const int seg = blockIdx.y, h = blockIdx.z;
   const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
@@ -176,64 +220,107 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_fwd_mfma(const AttnParams p)
   }
   const float c = p.scale * LOG2E;
 
-  for (int k0 = 0; k0 < L; k0 += BNK) {
+  TileStager<ND, BNK, G::PK, PIPE ? NT : BNK * G::CH> sk;  // (degenerate when not pipelined)
+  TileStager<ND, BNK, G::PV, PIPE ? NT : BNK * G::CH> sv;
+  if (PIPE) {
+    sk.init(p.k_stride);
+    sv.init(p.v_stride);
+    sk.load(K, min(BNK, L));
+    sv.load(V, min(BNK, L));
+    sk.store(lds_k[0]);
+    sv.store(lds_v[0]);
     __syncthreads();
-    const int valid = min(BNK, L - k0);
-    stage_tile<ND, G::PK, NT>(lds_k, K + (int64_t)k0 * p.k_stride, p.k_stride, BNK, valid);
-    stage_tile<ND, G::PV, NT>(lds_v, V + (int64_t)k0 * p.v_stride, p.v_stride, BNK, valid);
-    __syncthreads();
+  }
 
-    // scores: s[qb][kt][i] = S[query qb*16 + r][key kt*16 + 4g + i]
-    f32x4 s[4][4];
+  int buf = 0;
+  for (int k0 = 0; k0 < L; k0 += BNK) {
+    const int valid = min(BNK, L - k0);
+    const bool has_next = k0 + BNK < L;
+    if (PIPE) {
+      if (has_next) {
+        const int nv = min(BNK, L - k0 - BNK);
+        sk.load(K + (int64_t)(k0 + BNK) * p.k_stride, nv);
+        sv.load(V + (int64_t)(k0 + BNK) * p.v_stride, nv);
+      }
+    } else {
+      if (k0 > 0) __syncthreads();
+      stage_tile<ND, G::PK, NT>(lds_k[0], K + (int64_t)k0 * p.k_stride, p.k_stride, BNK, valid);
+      stage_tile<ND, G::PV, NT>(lds_v[0], V + (int64_t)k0 * p.v_stride, p.v_stride, BNK, valid);
+      __syncthreads();
+    }
+    const bf16_t* tk = lds_k[PIPE ? buf : 0];
+    const bf16_t* tv = lds_v[PIPE ? buf : 0];
+
+    // raw scores: s[qb][kt][i] = S[query qb*16 + r][key kt*16 + 4g + i]
+    f32x4 s[4][KT];
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt) {
+    for (int kt = 0; kt < KT; ++kt) {
       RowFrag<ND> kf;
-      load_rowfrag_lds<ND, G::PK>(kf, lds_k, kt * 16 + r, g);
+      load_rowfrag_lds<ND, G::PK>(kf, tk, kt * 16 + r, g);
 #pragma unroll
       for (int qb = 0; qb < 4; ++qb) s[qb][kt] = dot_frag<ND>(kf, qf[qb]);
     }
-    bf16x8 pb[4][2];
+    if (valid < BNK) {  // last, partial tile of the segment
+#pragma unroll
+      for (int qb = 0; qb < 4; ++qb)
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (kt * 16 + 4 * g + i >= valid) s[qb][kt][i] = -INFINITY;
+    }
+    bf16x8 pb[4][KK];
 #pragma unroll
     for (int qb = 0; qb < 4; ++qb) {
-      float mx = -INFINITY;
+      float mx = fmaxf(s[qb][0][0], s[qb][0][1]);
+      mx = max3(mx, s[qb][0][2], s[qb][0][3]);
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const bool ok = (kt * 16 + 4 * g + i) < valid;
-          s[qb][kt][i] = ok ? s[qb][kt][i] * c : -INFINITY;
-          mx = fmaxf(mx, s[qb][kt][i]);
-        }
+      for (int kt = 1; kt < KT; ++kt) {
+        mx = max3(mx, s[qb][kt][0], s[qb][kt][1]);
+        mx = max3(mx, s[qb][kt][2], s[qb][kt][3]);
+      }
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run[qb], mx);  // finite: every tile holds at least one valid key
-      const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_new);
-      m_run[qb] = m_new;
+      const float m_new = fmaxf(m_run[qb], mx * c);  // c > 0; finite: every tile holds at least one valid key
+      if (__builtin_amdgcn_ballot_w64(m_new > m_run[qb]) != 0) {
+        const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_new);
+        m_run[qb] = m_new;
+        l_run[qb] *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) o[qb][dt] *= alpha;
+      }
+      const float neg_m = -m_run[qb];
       float ps = 0.f;
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt)
+      for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float e = __builtin_amdgcn_exp2f(s[qb][kt][i] - m_new);
+          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][kt][i], c, neg_m));
           s[qb][kt][i] = e;
           ps += e;
         }
-      l_run[qb] = l_run[qb] * alpha + ps;
+      l_run[qb] += ps;
 #pragma unroll
-      for (int dt = 0; dt < ND; ++dt) o[qb][dt] *= alpha;
-      pb[qb][0] = pack8(s[qb][0], s[qb][1]);
-      pb[qb][1] = pack8(s[qb][2], s[qb][3]);
+      for (int kk = 0; kk < KK; ++kk) pb[qb][kk] = pack8(s[qb][2 * kk], s[qb][2 * kk + 1]);
     }
     // O^T[d][q] += sum_key V[key][d] P[q][key]; contraction slots (g, j): keys t0*16+4g+j | t1*16+4g+j-4
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk)
+    for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
       for (int dt = 0; dt < ND; ++dt) {
-        const bf16_t* a0 = lds_v + ((2 * kk) * 16 + 4 * g + (r >> 2)) * G::PV + 16 * dt + 4 * (r & 3);
+        const bf16_t* a0 = tv + ((2 * kk) * 16 + 4 * g + (r >> 2)) * G::PV + 16 * dt + 4 * (r & 3);
         const bf16x8 vf = tr_pair(a0, a0 + 16 * G::PV);
 #pragma unroll
         for (int qb = 0; qb < 4; ++qb) o[qb][dt] = mfma32(vf, pb[qb][kk], o[qb][dt]);
       }
+    if (PIPE) {
+      if (has_next) {
+        sk.store(lds_k[buf ^ 1]);
+        sv.store(lds_v[buf ^ 1]);
+      }
+      __syncthreads();
+      buf ^= 1;
+    }
   }
 
   bf16_t* O = static_cast<bf16_t*>(p.out) + (int64_t)s0 * p.o_stride + (int64_t)h * HD;
@@ -286,15 +373,16 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const T* __restrict__ o
 }
 
 // ================================================================================================
-// dK, dV.  Block = 64*NWAVES keys of one (segment, head); 32 queries per iteration.
+// dK, dV.  Block = 64*NWAVES keys of one (segment, head); 32 queries per iteration, Q / dO tiles (and the
+// rows' lse, delta) double buffered in LDS with the next tile's loads in flight during the MFMAs.
 template <int ND, int NWAVES>
 __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnParams p) {
   using G = Geo<ND>;
   constexpr int HD = G::HD, BQ = 32, NT = 64 * NWAVES;
-  __shared__ __attribute__((aligned(16))) bf16_t lds_q[BQ * G::PK];
-  __shared__ __attribute__((aligned(16))) bf16_t lds_do[BQ * G::PK];
-  __shared__ __attribute__((aligned(16))) float lds_lse[BQ];
-  __shared__ __attribute__((aligned(16))) float lds_delta[BQ];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_q[2][BQ * G::PK];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_do[2][BQ * G::PK];
+  __shared__ __attribute__((aligned(16))) float lds_lse[2][BQ];
+  __shared__ __attribute__((aligned(16))) float lds_delta[2][BQ];
 
   const int seg = blockIdx.y, h = blockIdx.z;
   const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
@@ -327,33 +415,58 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
     }
   const float c = p.scale * LOG2E;
 
-  for (int qs = 0; qs < L; qs += BQ) {
-    __syncthreads();
-    const int valid = min(BQ, L - qs);
-    stage_tile<ND, G::PK, NT>(lds_q, Q + (int64_t)qs * p.q_stride, p.q_stride, BQ, valid);
-    stage_tile<ND, G::PK, NT>(lds_do, DO + (int64_t)qs * p.do_stride, p.do_stride, BQ, valid);
+  TileStager<ND, BQ, G::PK, NT> sq, sdo;
+  sq.init(p.q_stride);
+  sdo.init(p.do_stride);
+  float r_lse = 0.f, r_delta = 0.f;  // threads 0..31 carry one row's statistics
+  auto load_stats = [&](int qs, int valid) {
     if (threadIdx.x < BQ) {
       const bool ok = (int)threadIdx.x < valid;
-      lds_lse[threadIdx.x] = ok ? LSE[qs + threadIdx.x] * LOG2E : INFINITY;  // +inf => p = 0 for padded queries
-      lds_delta[threadIdx.x] = ok ? DELTA[qs + threadIdx.x] : 0.f;
+      r_lse = ok ? LSE[qs + threadIdx.x] * LOG2E : INFINITY;  // +inf => p = 0 for padded queries
+      r_delta = ok ? DELTA[qs + threadIdx.x] : 0.f;
     }
-    __syncthreads();
+  };
+  auto store_stats = [&](int b) {
+    if (threadIdx.x < BQ) {
+      lds_lse[b][threadIdx.x] = r_lse;
+      lds_delta[b][threadIdx.x] = r_delta;
+    }
+  };
+  sq.load(Q, min(BQ, L));
+  sdo.load(DO, min(BQ, L));
+  load_stats(0, min(BQ, L));
+  sq.store(lds_q[0]);
+  sdo.store(lds_do[0]);
+  store_stats(0);
+  __syncthreads();
+
+  int buf = 0;
+  for (int qs = 0; qs < L; qs += BQ) {
+    const bool has_next = qs + BQ < L;
+    if (has_next) {
+      const int nv = min(BQ, L - qs - BQ);
+      sq.load(Q + (int64_t)(qs + BQ) * p.q_stride, nv);
+      sdo.load(DO + (int64_t)(qs + BQ) * p.do_stride, nv);
+      load_stats(qs + BQ, nv);
+    }
+    const bf16_t* tq = lds_q[buf];
+    const bf16_t* tdo = lds_do[buf];
 
     RowFrag<ND> qa[2], da[2];  // natural-layout A operands: row = query t*16 + r
     bf16x8 qt[ND], dt_[ND];    // transposed A operands: row = head-dim 16*dt + r, slots = queries
     f32x4 lse2[2], dl[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      load_rowfrag_lds<ND, G::PK>(qa[t], lds_q, t * 16 + r, g);
-      load_rowfrag_lds<ND, G::PK>(da[t], lds_do, t * 16 + r, g);
-      lse2[t] = *reinterpret_cast<const f32x4*>(lds_lse + t * 16 + 4 * g);
-      dl[t] = *reinterpret_cast<const f32x4*>(lds_delta + t * 16 + 4 * g);
+      load_rowfrag_lds<ND, G::PK>(qa[t], tq, t * 16 + r, g);
+      load_rowfrag_lds<ND, G::PK>(da[t], tdo, t * 16 + r, g);
+      lse2[t] = *reinterpret_cast<const f32x4*>(lds_lse[buf] + t * 16 + 4 * g);
+      dl[t] = *reinterpret_cast<const f32x4*>(lds_delta[buf] + t * 16 + 4 * g);
     }
 #pragma unroll
     for (int d = 0; d < ND; ++d) {
       const int off = (4 * g + (r >> 2)) * G::PK + 16 * d + 4 * (r & 3);
-      qt[d] = tr_pair(lds_q + off, lds_q + off + 16 * G::PK);
-      dt_[d] = tr_pair(lds_do + off, lds_do + off + 16 * G::PK);
+      qt[d] = tr_pair(tq + off, tq + off + 16 * G::PK);
+      dt_[d] = tr_pair(tdo + off, tdo + off + 16 * G::PK);
     }
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
@@ -364,7 +477,7 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
         const f32x4 dp = dot_frag<ND>(da[t], vf[kb]);  // dP, same layout
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float e = __builtin_amdgcn_exp2f(s[i] * c - lse2[t][i]);
+          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c, -lse2[t][i]));
           pv[t][i] = e;
           ds[t][i] = e * (dp[i] - dl[t][i]);
         }
@@ -377,6 +490,13 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
         dk[kb][d] = mfma32(qt[d], dsb, dk[kb][d]);
       }
     }
+    if (has_next) {
+      sq.store(lds_q[buf ^ 1]);
+      sdo.store(lds_do[buf ^ 1]);
+      store_stats(buf ^ 1);
+    }
+    __syncthreads();
+    buf ^= 1;
   }
 
   bf16_t* DK = static_cast<bf16_t*>(p.dk) + (int64_t)s0 * p.dk_stride + (int64_t)h * HD;
@@ -401,13 +521,13 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
 }
 
 // ================================================================================================
-// dQ.  Block = 64*NWAVES queries of one (segment, head); 32 keys per iteration.
+// dQ.  Block = 64*NWAVES queries of one (segment, head); 32 keys per iteration, K / V tiles double buffered.
 template <int ND, int NWAVES>
 __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams p) {
   using G = Geo<ND>;
   constexpr int HD = G::HD, BK = 32, NT = 64 * NWAVES;
-  __shared__ __attribute__((aligned(16))) bf16_t lds_k[BK * G::PK];
-  __shared__ __attribute__((aligned(16))) bf16_t lds_v[BK * G::PK];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_k[2][BK * G::PK];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_v[2][BK * G::PK];
 
   const int seg = blockIdx.y, h = blockIdx.z;
   const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
@@ -424,14 +544,14 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams
   const float* DELTA = p.delta + (int64_t)h * p.total + s0;
 
   RowFrag<ND> qf[4], dof[4];
-  float lse2[4], dl[4];
+  float neg_lse2[4], dl[4];
 #pragma unroll
   for (int qb = 0; qb < 4; ++qb) {
     const int qi = q0 + qb * 16 + r;
     const bool ok = qi < L;
     load_rowfrag_global<ND>(qf[qb], Q + (int64_t)qi * p.q_stride, ok, g);
     load_rowfrag_global<ND>(dof[qb], DO + (int64_t)qi * p.do_stride, ok, g);
-    lse2[qb] = ok ? LSE[qi] * LOG2E : INFINITY;
+    neg_lse2[qb] = ok ? -LSE[qi] * LOG2E : -INFINITY;
     dl[qb] = ok ? DELTA[qi] : 0.f;
   }
   f32x4 dq[4][ND];
@@ -441,24 +561,38 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams
     for (int d = 0; d < ND; ++d) dq[qb][d] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float c = p.scale * LOG2E;
 
+  TileStager<ND, BK, G::PK, NT> sk, sv;
+  sk.init(p.k_stride);
+  sv.init(p.v_stride);
+  sk.load(K, min(BK, L));
+  sv.load(V, min(BK, L));
+  sk.store(lds_k[0]);
+  sv.store(lds_v[0]);
+  __syncthreads();
+
+  int buf = 0;
   for (int k0 = 0; k0 < L; k0 += BK) {
-    __syncthreads();
     const int valid = min(BK, L - k0);
-    stage_tile<ND, G::PK, NT>(lds_k, K + (int64_t)k0 * p.k_stride, p.k_stride, BK, valid);
-    stage_tile<ND, G::PK, NT>(lds_v, V + (int64_t)k0 * p.v_stride, p.v_stride, BK, valid);
-    __syncthreads();
+    const bool has_next = k0 + BK < L;
+    if (has_next) {
+      const int nv = min(BK, L - k0 - BK);
+      sk.load(K + (int64_t)(k0 + BK) * p.k_stride, nv);
+      sv.load(V + (int64_t)(k0 + BK) * p.v_stride, nv);
+    }
+    const bf16_t* tk = lds_k[buf];
+    const bf16_t* tv = lds_v[buf];
 
     RowFrag<ND> ka[2], va[2];
     bf16x8 kt[ND];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      load_rowfrag_lds<ND, G::PK>(ka[t], lds_k, t * 16 + r, g);
-      load_rowfrag_lds<ND, G::PK>(va[t], lds_v, t * 16 + r, g);
+      load_rowfrag_lds<ND, G::PK>(ka[t], tk, t * 16 + r, g);
+      load_rowfrag_lds<ND, G::PK>(va[t], tv, t * 16 + r, g);
     }
 #pragma unroll
     for (int d = 0; d < ND; ++d) {
       const int off = (4 * g + (r >> 2)) * G::PK + 16 * d + 4 * (r & 3);
-      kt[d] = tr_pair(lds_k + off, lds_k + off + 16 * G::PK);
+      kt[d] = tr_pair(tk + off, tk + off + 16 * G::PK);
     }
 #pragma unroll
     for (int qb = 0; qb < 4; ++qb) {
@@ -469,15 +603,27 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams
         const f32x4 dp = dot_frag<ND>(va[t], dof[qb]);  // dP, same layout
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const bool ok = (t * 16 + 4 * g + i) < valid;
-          const float e = ok ? __builtin_amdgcn_exp2f(s[i] * c - lse2[qb]) : 0.f;
+          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c, neg_lse2[qb]));
           ds[t][i] = e * (dp[i] - dl[qb]);
         }
+      }
+      if (valid < BK) {  // keys past the segment end contribute nothing
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (t * 16 + 4 * g + i >= valid) ds[t][i] = 0.f;
       }
       const bf16x8 dsb = pack8(ds[0], ds[1]);
 #pragma unroll
       for (int d = 0; d < ND; ++d) dq[qb][d] = mfma32(kt[d], dsb, dq[qb][d]);
     }
+    if (has_next) {
+      sk.store(lds_k[buf ^ 1]);
+      sv.store(lds_v[buf ^ 1]);
+    }
+    __syncthreads();
+    buf ^= 1;
   }
 
   bf16_t* DQ = static_cast<bf16_t*>(p.dq) + (int64_t)s0 * p.dq_stride + (int64_t)h * HD;
@@ -685,9 +831,9 @@ template <int ND>
 int launch_fwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t s) {
   const int nw = pick_waves(max_seqlen);
   dim3 grid((unsigned)((max_seqlen + 64 * nw - 1) / (64 * nw)), (unsigned)n_seg, (unsigned)p.nheads);
-  if (nw == 1) hipLaunchKernelGGL((attn_fwd_mfma<ND, 1>), grid, 64, 0, s, p);
-  else if (nw == 2) hipLaunchKernelGGL((attn_fwd_mfma<ND, 2>), grid, 128, 0, s, p);
-  else hipLaunchKernelGGL((attn_fwd_mfma<ND, 4>), grid, 256, 0, s, p);
+  if (nw == 1) hipLaunchKernelGGL((attn_fwd_mfma<ND, 1, 64, false>), grid, 64, 0, s, p);
+  else if (nw == 2) hipLaunchKernelGGL((attn_fwd_mfma<ND, 2, 64, false>), grid, 128, 0, s, p);
+  else hipLaunchKernelGGL((attn_fwd_mfma<ND, 4, 32, true>), grid, 256, 0, s, p);
   MVIT_CHECK_LAUNCH("attn_fwd");
   return MVIT_OK;
 }

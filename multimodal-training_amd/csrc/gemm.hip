@@ -1,20 +1,23 @@
 // MFMA GEMM for gfx950 with fused epilogues:  C[M,N] = epi( sum_k A[m,k] * B[n,k] ).
 //
-// Block tile 256x128 (M x N), 4 waves in a 2x2 grid, each wave owning 128x64 as 4x2 MFMA 32x32 tiles.
+// Block tile 256x256.  Two wave layouts are built (selected by the host per problem):
+//   V0: 4 waves (2x2), each owning 128x128 as 4x4 MFMA 32x32 tiles (least LDS traffic per FLOP);
+//   V1: 8 waves (2x4), each owning 128x64  as 4x2 tiles (two waves per SIMD hide each other's LDS latency).
 //   bf16: v_mfma_f32_32x32x16_bf16, BK = 64.  Operands whose contraction index is contiguous in memory are
 //         staged as [row][k] and read with 16-byte LDS loads; operands whose contraction index is the slow
 //         dimension (dgrad's weight, both operands of wgrad) are staged as [k][row] exactly as they lie in
 //         memory and read with ds_read_b64_tr_b16, which hands each lane 4 consecutive k for its row.
 //   fp32: v_mfma_f32_32x32x2_f32, BK = 16 (parity mode; one LDS word per lane per MFMA operand).
-// The next K tile is fetched into registers while the current one is consumed from LDS.
+// LDS is double buffered: the next K tile travels global -> registers while the current one is consumed,
+// is written to the other buffer after the MFMAs, and one barrier per K step separates the two.
+// The epilogue stages the accumulators through LDS (fp32) so that bias / residual / activation inputs are
+// read and results written as 16-byte vectors along N.
 // Work-group ids are remapped so that the tiles a single XCD (one L2) works on are neighbours in N.
 #include "mvit_common.h"
 
 namespace {
 
-constexpr int BM = 256, BN = 128;
-constexpr int WAVE_M = 128, WAVE_N = 64;  // per-wave tile
-constexpr int MT = WAVE_M / 32, NT = WAVE_N / 32;
+constexpr int BM = 256, BN = 256;
 
 struct GemmParams {
   int64_t M, N, K;
@@ -36,6 +39,7 @@ struct GemmParams {
   int split_k;        // K slices (1 = none)
   int64_t k_chunk;    // K extent of one slice (multiple of BK)
   float* workspace;   // [split_k][M][N] fp32 partial sums when split_k > 1
+  int vec_ok;         // every epilogue pointer / stride allows 16-byte accesses
 };
 
 template <typename T>
@@ -53,6 +57,17 @@ struct Cfg<float> {
   static constexpr int PAD_T = 4;
 };
 
+template <int VAR>
+struct Waves;
+template <>
+struct Waves<0> {
+  static constexpr int WM = 128, WN = 128, NTHREADS = 256;
+};
+template <>
+struct Waves<1> {
+  static constexpr int WM = 128, WN = 64, NTHREADS = 512;
+};
+
 __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.f + erff(z * 0.70710678118654752440f)); }
 __device__ __forceinline__ float gelu_erf_grad(float z) {
   const float cdf = 0.5f * (1.f + erff(z * 0.70710678118654752440f));
@@ -61,24 +76,51 @@ __device__ __forceinline__ float gelu_erf_grad(float z) {
 }
 __device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + __expf(-z)); }
 
-// Stage one operand tile (ROWS rows of the output dimension x BK of the contraction) global -> registers.
+// 8 consecutive elements <-> fp32 registers
+__device__ __forceinline__ void load8(const bf16_t* p, float* v) {
+  const bf16x8 x = *reinterpret_cast<const bf16x8*>(p);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = (float)x[e];
+}
+__device__ __forceinline__ void load8(const float* p, float* v) {
+  const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    v[e] = a[e];
+    v[4 + e] = b[e];
+  }
+}
+__device__ __forceinline__ void store8(bf16_t* p, const float* v) {
+  bf16x8 x;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) x[e] = (bf16_t)v[e];
+  *reinterpret_cast<bf16x8*>(p) = x;
+}
+__device__ __forceinline__ void store8(float* p, const float* v) {
+  *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]};
+  *reinterpret_cast<f32x4*>(p + 4) = f32x4{v[4], v[5], v[6], v[7]};
+}
+
+// Stage one operand tile (ROWS rows of the output dimension x BK of the contraction) global -> registers -> LDS.
 // TR = false: memory is [row][k];  TR = true: memory is [k][row].
-template <typename T, int ROWS, bool TR>
+template <typename T, int ROWS, bool TR, int NTHREADS, int WN>
 struct TileLoader {
   using C = Cfg<T>;
   static constexpr int V = C::VEC;
   typedef T vec_t __attribute__((ext_vector_type(V)));
   static constexpr int CHUNKS = ROWS * C::BK / V;  // 16-byte chunks per tile
-  static constexpr int PER_THREAD = CHUNKS / 256;
+  static constexpr int PER_THREAD = CHUNKS / NTHREADS;
   static constexpr int LDS_ELEMS = TR ? C::BK * (ROWS + C::PAD_T) : ROWS * C::PITCH_K;
   vec_t regs[PER_THREAD];
 
-  // row_map: SWIGLU packs two weight matrices into one B tile; otherwise identity.
+  // dual: SWIGLU packs two weight matrices into one B tile so that a wave's first N sub-tiles are gate columns and
+  // its last ones the up columns with the same indices: tile row r = wn*WN + half*(WN/2) + j -> matrix `half`,
+  // row row0 + wn*(WN/2) + j.
   __device__ __forceinline__ void load(const T* __restrict__ base, const T* __restrict__ base2, int64_t ld,
-                                       int64_t row0, int64_t row_limit, int64_t k0, int64_t K, bool dual) {
+                                       int64_t row0, int64_t row_limit, int64_t k0, int64_t k_end, bool dual) {
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
-      const int c = threadIdx.x + 256 * i;
+      const int c = threadIdx.x + NTHREADS * i;
       int r, kk;
       if (!TR) {
         r = c / (C::BK / V);
@@ -90,9 +132,8 @@ struct TileLoader {
       const T* src = base;
       int64_t grow;
       if (dual) {
-        // tile row r = wn*64 + half*32 + j  ->  matrix `half`, row row0 + wn*32 + j   (ROWS == 128, !TR)
-        const int wn = r >> 6, half = (r >> 5) & 1, j = r & 31;
-        grow = row0 + wn * 32 + j;
+        const int wn = r / WN, w = r % WN, half = w / (WN / 2), j = w % (WN / 2);
+        grow = row0 + wn * (WN / 2) + j;
         if (half) src = base2;
       } else {
         grow = row0 + r;
@@ -102,9 +143,9 @@ struct TileLoader {
 #pragma unroll
       for (int j = 0; j < V; ++j) v[j] = from_f32<T>(0.f);
       if (!TR) {
-        if (grow < row_limit && gk < K) v = *reinterpret_cast<const vec_t*>(src + grow * ld + gk);
+        if (grow < row_limit && gk < k_end) v = *reinterpret_cast<const vec_t*>(src + grow * ld + gk);
       } else {
-        if (grow < row_limit && gk < K) v = *reinterpret_cast<const vec_t*>(src + gk * ld + grow);
+        if (grow < row_limit && gk < k_end) v = *reinterpret_cast<const vec_t*>(src + gk * ld + grow);
       }
       regs[i] = v;
     }
@@ -112,7 +153,7 @@ struct TileLoader {
   __device__ __forceinline__ void store(T* lds) const {
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
-      const int c = threadIdx.x + 256 * i;
+      const int c = threadIdx.x + NTHREADS * i;
       int off;
       if (!TR) {
         const int r = c / (C::BK / V), kk = (c % (C::BK / V)) * V;
@@ -158,15 +199,132 @@ __device__ __forceinline__ float frag_f32(const float* lds, int row, int k) {
     return lds[(k + (l >> 5)) * (ROWS + C::PAD_T) + row + (l & 31)];
 }
 
-template <typename T, typename TO, bool TA, bool TB, int EPI>
-__global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
+// Epilogue on 8 consecutive output columns n..n+7 of row m.  v: accumulators (gate half for SWIGLU), u: up half.
+template <typename T, typename TO, int EPI>
+__device__ __forceinline__ void emit8(const GemmParams& p, int64_t m, int64_t n, float* v, const float* u, bool vec) {
+  TO* Cp = static_cast<TO*>(p.C);
+  const T* Rp = static_cast<const T*>(p.R);
+  T* auxp = static_cast<T*>(p.aux);
+  const T* bias = static_cast<const T*>(p.bias);
+  const T* bias2 = static_cast<const T*>(p.bias2);
+  const int cnt = (p.N - n) < 8 ? (int)(p.N - n) : 8;
+  vec = vec && cnt == 8;
+
+  if constexpr (EPI == MVIT_EPI_BIAS || EPI == MVIT_EPI_BIAS_RES || EPI == MVIT_EPI_BIAS_GELU || EPI == MVIT_EPI_SWIGLU) {
+    if (bias) {
+      float b[8];
+      if (vec) load8(bias + n, b);
+      else
+        for (int e = 0; e < cnt; ++e) b[e] = to_f32(bias[n + e]);
+      for (int e = 0; e < cnt; ++e) v[e] += b[e];
+    }
+  }
+  if constexpr (EPI == MVIT_EPI_SWIGLU) {
+    float uu[8], h[8];
+    for (int e = 0; e < 8; ++e) uu[e] = u[e];
+    if (bias2) {
+      float b[8];
+      if (vec) load8(bias2 + n, b);
+      else
+        for (int e = 0; e < cnt; ++e) b[e] = to_f32(bias2[n + e]);
+      for (int e = 0; e < cnt; ++e) uu[e] += b[e];
+    }
+    // round g and u to the storage type first: the backward recomputes from those stored values
+    for (int e = 0; e < 8; ++e) {
+      v[e] = to_f32(from_f32<T>(v[e]));
+      uu[e] = to_f32(from_f32<T>(uu[e]));
+      h[e] = v[e] * sigmoidf_(v[e]) * uu[e];
+    }
+    T* g_out = auxp + m * p.ldaux + n;
+    T* u_out = g_out + p.aux_off;
+    TO* h_out = Cp + m * p.ldc + n;
+    if (vec) {
+      store8(g_out, v);
+      store8(u_out, uu);
+      store8(h_out, h);
+    } else {
+      for (int e = 0; e < cnt; ++e) {
+        g_out[e] = from_f32<T>(v[e]);
+        u_out[e] = from_f32<T>(uu[e]);
+        h_out[e] = from_f32<TO>(h[e]);
+      }
+    }
+    return;
+  }
+  if constexpr (EPI == MVIT_EPI_SWIGLU_BWD) {
+    const T* g_in = Rp + m * p.ldr + n;
+    const T* u_in = g_in + p.aux_off;
+    float g[8], uu[8], dg[8], du[8];
+    if (vec) {
+      load8(g_in, g);
+      load8(u_in, uu);
+    } else {
+      for (int e = 0; e < 8; ++e) {
+        g[e] = e < cnt ? to_f32(g_in[e]) : 0.f;
+        uu[e] = e < cnt ? to_f32(u_in[e]) : 0.f;
+      }
+    }
+    for (int e = 0; e < 8; ++e) {
+      const float sg = sigmoidf_(g[e]);
+      const float silu = g[e] * sg;
+      dg[e] = v[e] * uu[e] * (sg + silu * (1.f - sg));
+      du[e] = v[e] * silu;
+    }
+    TO* dg_out = Cp + m * p.ldc + n;
+    TO* du_out = dg_out + p.aux_off;
+    if (vec) {
+      store8(dg_out, dg);
+      store8(du_out, du);
+    } else {
+      for (int e = 0; e < cnt; ++e) {
+        dg_out[e] = from_f32<TO>(dg[e]);
+        du_out[e] = from_f32<TO>(du[e]);
+      }
+    }
+    return;
+  }
+  if constexpr (EPI == MVIT_EPI_BIAS_RES || EPI == MVIT_EPI_GELU_BWD) {
+    float r[8];
+    if (vec) load8(Rp + m * p.ldr + n, r);
+    else
+      for (int e = 0; e < 8; ++e) r[e] = e < cnt ? to_f32(Rp[m * p.ldr + n + e]) : 0.f;
+    for (int e = 0; e < 8; ++e) {
+      if constexpr (EPI == MVIT_EPI_BIAS_RES) v[e] += r[e];
+      else v[e] *= gelu_erf_grad(r[e]);
+    }
+  }
+  if constexpr (EPI == MVIT_EPI_BIAS_GELU) {
+    T* z_out = auxp + m * p.ldaux + n;
+    for (int e = 0; e < 8; ++e) v[e] = to_f32(from_f32<T>(v[e]));  // gelu of the stored pre-activation
+    if (vec) store8(z_out, v);
+    else
+      for (int e = 0; e < cnt; ++e) z_out[e] = from_f32<T>(v[e]);
+    for (int e = 0; e < 8; ++e) v[e] = gelu_erf(v[e]);
+  }
+  TO* c_out = Cp + m * p.ldc + n;
+  if constexpr (EPI == MVIT_EPI_ACCUM) {
+    float c[8];
+    if (vec) load8(c_out, c);
+    else
+      for (int e = 0; e < 8; ++e) c[e] = e < cnt ? to_f32(c_out[e]) : 0.f;
+    for (int e = 0; e < 8; ++e) v[e] += c[e];
+  }
+  if (vec) store8(c_out, v);
+  else
+    for (int e = 0; e < cnt; ++e) c_out[e] = from_f32<TO>(v[e]);
+}
+
+template <typename T, typename TO, bool TA, bool TB, int EPI, int VAR>
+__global__ __launch_bounds__(Waves<VAR>::NTHREADS) void gemm_kernel(const GemmParams p) {
   using C = Cfg<T>;
-  constexpr int BK = C::BK;
-  using LoaderA = TileLoader<T, BM, TA>;
-  using LoaderB = TileLoader<T, BN, TB>;
+  using W = Waves<VAR>;
+  constexpr int BK = C::BK, WM = W::WM, WN = W::WN, NTHREADS = W::NTHREADS;
+  constexpr int MT = WM / 32, NT = WN / 32, WGN = BN / WN;  // waves along N
+  using LoaderA = TileLoader<T, BM, TA, NTHREADS, WN>;
+  using LoaderB = TileLoader<T, BN, TB, NTHREADS, WN>;
+  constexpr int STAGE_ELEMS = LoaderA::LDS_ELEMS + LoaderB::LDS_ELEMS;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  T* lds_a = reinterpret_cast<T*>(smem_raw);
-  T* lds_b = lds_a + LoaderA::LDS_ELEMS;
+  T* lds = reinterpret_cast<T*>(smem_raw);
 
   // XCD-aware tile order: hardware deals consecutive work-group ids round-robin to the 8 XCDs; give each
   // XCD a contiguous range of tiles (N fastest) so that its L2 sees one A panel at a time.
@@ -185,7 +343,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
   const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * N_PER_BLOCK;
 
   const int l = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int wm = wv >> 1, wn = wv & 1;
+  const int wm = wv / WGN, wn = wv % WGN;
 
   f32x16 acc[MT][NT];
 #pragma unroll
@@ -202,24 +360,27 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
   const T* B2 = static_cast<const T*>(p.B2);
   la.load(A, nullptr, p.lda, m0, p.M, k_begin, k_end, false);
   lb.load(B, B2, p.ldb, n0, p.N, k_begin, k_end, DUAL);
+  la.store(lds);
+  lb.store(lds + LoaderA::LDS_ELEMS);
+  __syncthreads();
 
+  int buf = 0;
   for (int64_t k0 = k_begin; k0 < k_end; k0 += BK) {
-    __syncthreads();  // previous tile fully consumed
-    la.store(lds_a);
-    lb.store(lds_b);
-    __syncthreads();
-    if (k0 + BK < k_end) {
+    const bool has_next = k0 + BK < k_end;
+    if (has_next) {
       la.load(A, nullptr, p.lda, m0, p.M, k0 + BK, k_end, false);
       lb.load(B, B2, p.ldb, n0, p.N, k0 + BK, k_end, DUAL);
     }
+    const T* lds_a = lds + buf * STAGE_ELEMS;
+    const T* lds_b = lds_a + LoaderA::LDS_ELEMS;
     if constexpr (sizeof(T) == 2) {
 #pragma unroll
       for (int ks = 0; ks < BK; ks += 16) {
         bf16x8 fa[MT], fb[NT];
 #pragma unroll
-        for (int a = 0; a < MT; ++a) fa[a] = frag_bf16<TA, BM>(reinterpret_cast<const bf16_t*>(lds_a), wm * WAVE_M + a * 32, ks);
+        for (int a = 0; a < MT; ++a) fa[a] = frag_bf16<TA, BM>(reinterpret_cast<const bf16_t*>(lds_a), wm * WM + a * 32, ks);
 #pragma unroll
-        for (int b = 0; b < NT; ++b) fb[b] = frag_bf16<TB, BN>(reinterpret_cast<const bf16_t*>(lds_b), wn * WAVE_N + b * 32, ks);
+        for (int b = 0; b < NT; ++b) fb[b] = frag_bf16<TB, BN>(reinterpret_cast<const bf16_t*>(lds_b), wn * WN + b * 32, ks);
 #pragma unroll
         for (int a = 0; a < MT; ++a)
 #pragma unroll
@@ -230,105 +391,79 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
       for (int ks = 0; ks < BK; ks += 2) {
         float fa[MT], fb[NT];
 #pragma unroll
-        for (int a = 0; a < MT; ++a) fa[a] = frag_f32<TA, BM>(reinterpret_cast<const float*>(lds_a), wm * WAVE_M + a * 32, ks);
+        for (int a = 0; a < MT; ++a) fa[a] = frag_f32<TA, BM>(reinterpret_cast<const float*>(lds_a), wm * WM + a * 32, ks);
 #pragma unroll
-        for (int b = 0; b < NT; ++b) fb[b] = frag_f32<TB, BN>(reinterpret_cast<const float*>(lds_b), wn * WAVE_N + b * 32, ks);
+        for (int b = 0; b < NT; ++b) fb[b] = frag_f32<TB, BN>(reinterpret_cast<const float*>(lds_b), wn * WN + b * 32, ks);
 #pragma unroll
         for (int a = 0; a < MT; ++a)
 #pragma unroll
           for (int b = 0; b < NT; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a], fb[b], acc[a][b], 0, 0, 0);
       }
     }
+    if (has_next) {
+      T* nxt = lds + (buf ^ 1) * STAGE_ELEMS;
+      la.store(nxt);
+      lb.store(nxt + LoaderA::LDS_ELEMS);
+    }
+    __syncthreads();
+    buf ^= 1;
   }
 
-  // ---- epilogue.  acc[a][b][4*j+i] is C[m0 + wm*128 + a*32 + 8*j + 4*(l/32) + i][n-tile b, column l%32].
-  TO* Cp = static_cast<TO*>(p.C);
-  const T* Rp = static_cast<const T*>(p.R);
-  T* auxp = static_cast<T*>(p.aux);
-  const T* bias = static_cast<const T*>(p.bias);
-  const T* bias2 = static_cast<const T*>(p.bias2);
+  // ---- epilogue.  acc[a][b][4*j+i] is C[m0 + wm*WM + a*32 + 8*j + 4*(l/32) + i][wave column b*32 + l%32].
+  // Pass a: every wave parks its a-th 32-row sub-tile in LDS (fp32, [ (BM/WM)*32 rows ][ BN + 8 ]), then the block
+  // walks the pass in 8-column groups.
+  constexpr int SP = BN + 8;
+  constexpr int PASS_ROWS = (BM / WM) * 32;
+  constexpr int NCOLS = DUAL ? BN / 2 : BN;
+  constexpr int GROUPS = NCOLS / 8;
+  float* stage = reinterpret_cast<float*>(smem_raw);
   const int lc = l & 31, lr = 4 * (l >> 5);
-
-  if constexpr (EPI == MVIT_EPI_NONE) {
-    if (p.split_k > 1) {  // fp32 partial tile; summed over slices by splitk_reduce_kernel
-      float* W = p.workspace + (int64_t)slice * p.M * p.N;
+  const bool to_ws = (EPI == MVIT_EPI_NONE) && p.split_k > 1;
+  float* ws = to_ws ? p.workspace + (int64_t)slice * p.M * p.N : nullptr;
+  const bool ws_vec = (p.N % 4 == 0);
 #pragma unroll
-      for (int b = 0; b < NT; ++b) {
-        const int64_t n = n0 + wn * WAVE_N + b * 32 + lc;
-        if (n >= p.N) continue;
-#pragma unroll
-        for (int a = 0; a < MT; ++a)
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int64_t m = m0 + wm * WAVE_M + a * 32 + 8 * j + lr + i;
-              if (m < p.M) W[m * p.N + n] = acc[a][b][4 * j + i];
-            }
-      }
-      return;
-    }
-  }
-  if constexpr (DUAL) {
-    const int64_t n = n0 + wn * 32 + lc;
-    if (n < p.N) {
-      const float bg = bias ? to_f32(bias[n]) : 0.f, bu = bias2 ? to_f32(bias2[n]) : 0.f;
-#pragma unroll
-      for (int a = 0; a < MT; ++a)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int64_t m = m0 + wm * WAVE_M + a * 32 + 8 * j + lr + i;
-            if (m < p.M) {
-              // round g and u to the storage type first: the backward recomputes from those stored values
-              const T gs = from_f32<T>(acc[a][0][4 * j + i] + bg);
-              const T us = from_f32<T>(acc[a][1][4 * j + i] + bu);
-              auxp[m * p.ldaux + n] = gs;
-              auxp[m * p.ldaux + p.aux_off + n] = us;
-              const float g = to_f32(gs), u = to_f32(us);
-              Cp[m * p.ldc + n] = from_f32<TO>(g * sigmoidf_(g) * u);
-            }
-          }
-    }
-  } else {
+  for (int a = 0; a < MT; ++a) {
+    if (a > 0) __syncthreads();
 #pragma unroll
     for (int b = 0; b < NT; ++b) {
-      const int64_t n = n0 + wn * WAVE_N + b * 32 + lc;
-      if (n >= p.N) continue;
-      float bv = 0.f;
-      if constexpr (EPI == MVIT_EPI_BIAS || EPI == MVIT_EPI_BIAS_RES || EPI == MVIT_EPI_BIAS_GELU)
-        bv = bias ? to_f32(bias[n]) : 0.f;
+      int col;
+      if (DUAL) col = (b / (NT / 2)) * (BN / 2) + wn * (WN / 2) + (b % (NT / 2)) * 32 + lc;
+      else col = wn * WN + b * 32 + lc;
 #pragma unroll
-      for (int a = 0; a < MT; ++a)
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int i = 0; i < 4; ++i) stage[(wm * 32 + 8 * j + lr + i) * SP + col] = acc[a][b][4 * j + i];
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < PASS_ROWS * GROUPS; c += NTHREADS) {
+      const int row = c / GROUPS, cg = c % GROUPS;
+      const int64_t m = m0 + (row / 32) * WM + a * 32 + (row % 32);
+      const int64_t n = n0 + cg * 8;
+      if (m >= p.M || n >= p.N) continue;
+      float v[8], u[8];
+      const float* sp = stage + row * SP + cg * 8;
+      const f32x4 v0 = *reinterpret_cast<const f32x4*>(sp), v1 = *reinterpret_cast<const f32x4*>(sp + 4);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int64_t m = m0 + wm * WAVE_M + a * 32 + 8 * j + lr + i;
-            if (m >= p.M) continue;
-            float v = acc[a][b][4 * j + i] + bv;
-            if constexpr (EPI == MVIT_EPI_BIAS_RES) {
-              v += to_f32(Rp[m * p.ldr + n]);
-            } else if constexpr (EPI == MVIT_EPI_BIAS_GELU) {
-              const T zs = from_f32<T>(v);
-              auxp[m * p.ldaux + n] = zs;
-              v = gelu_erf(to_f32(zs));
-            } else if constexpr (EPI == MVIT_EPI_GELU_BWD) {
-              v *= gelu_erf_grad(to_f32(Rp[m * p.ldr + n]));
-            } else if constexpr (EPI == MVIT_EPI_ACCUM) {
-              v += to_f32(Cp[m * p.ldc + n]);
-            }
-            if constexpr (EPI == MVIT_EPI_SWIGLU_BWD) {
-              const float g = to_f32(Rp[m * p.ldr + n]), u = to_f32(Rp[m * p.ldr + p.aux_off + n]);
-              const float sg = sigmoidf_(g);
-              const float silu = g * sg;
-              Cp[m * p.ldc + n] = from_f32<TO>(v * u * (sg + silu * (1.f - sg)));
-              Cp[m * p.ldc + p.aux_off + n] = from_f32<TO>(v * silu);
-            } else {
-              Cp[m * p.ldc + n] = from_f32<TO>(v);
-            }
-          }
+      for (int e = 0; e < 4; ++e) {
+        v[e] = v0[e];
+        v[4 + e] = v1[e];
+      }
+      if (DUAL) {
+        const f32x4 u0 = *reinterpret_cast<const f32x4*>(sp + BN / 2), u1 = *reinterpret_cast<const f32x4*>(sp + BN / 2 + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          u[e] = u0[e];
+          u[4 + e] = u1[e];
+        }
+      }
+      if (to_ws) {
+        float* w = ws + m * p.N + n;
+        if (ws_vec && n + 8 <= p.N) store8(w, v);
+        else
+          for (int e = 0; e < 8 && n + e < p.N; ++e) w[e] = v[e];
+      } else {
+        emit8<T, TO, EPI>(p, m, n, v, u, p.vec_ok != 0);
+      }
     }
   }
 }
@@ -345,12 +480,15 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   }
 }
 
-template <typename T, typename TO, bool TA, bool TB, int EPI>
+template <typename T, typename TO, bool TA, bool TB, int EPI, int VAR>
 int launch(const GemmParams& p, hipStream_t stream) {
-  using LA = TileLoader<T, BM, TA>;
-  using LB = TileLoader<T, BN, TB>;
-  const size_t lds = (size_t)(LA::LDS_ELEMS + LB::LDS_ELEMS) * sizeof(T);
-  auto kern = gemm_kernel<T, TO, TA, TB, EPI>;
+  using W = Waves<VAR>;
+  using LA = TileLoader<T, BM, TA, W::NTHREADS, W::WN>;
+  using LB = TileLoader<T, BN, TB, W::NTHREADS, W::WN>;
+  const size_t operands = 2 * (size_t)(LA::LDS_ELEMS + LB::LDS_ELEMS) * sizeof(T);
+  const size_t staging = (size_t)(BM / W::WM) * 32 * (BN + 8) * sizeof(float);
+  const size_t lds = operands > staging ? operands : staging;
+  auto kern = gemm_kernel<T, TO, TA, TB, EPI, VAR>;
   static bool attr_set = false;  // dynamic LDS above 64 KiB needs opting in once per kernel
   if (!attr_set && lds > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -360,7 +498,7 @@ int launch(const GemmParams& p, hipStream_t stream) {
   if (p.split_k > 1 && EPI != MVIT_EPI_NONE) return mvit_set_error(MVIT_ERR_UNSUPPORTED, "gemm: split_k needs EPI_NONE");
   const int total = p.tiles_m * p.tiles_n * p.split_k;
   const int grid = ((total + 7) / 8) * 8;
-  hipLaunchKernelGGL(kern, grid, 256, lds, stream, p);
+  hipLaunchKernelGGL(kern, grid, W::NTHREADS, lds, stream, p);
   MVIT_CHECK_LAUNCH("gemm");
   if (p.split_k > 1) {
     const int64_t elems = p.M * p.N;
@@ -371,28 +509,34 @@ int launch(const GemmParams& p, hipStream_t stream) {
   return MVIT_OK;
 }
 
+template <typename T, typename TO, bool TA, bool TB, int EPI>
+int launch_var(int var, const GemmParams& p, hipStream_t s) {
+  if (var == 1) return launch<T, TO, TA, TB, EPI, 1>(p, s);
+  return launch<T, TO, TA, TB, EPI, 0>(p, s);
+}
+
 template <typename T, typename TO, bool TA, bool TB>
-int dispatch_epi(int epi, const GemmParams& p, hipStream_t s) {
+int dispatch_epi(int epi, int var, const GemmParams& p, hipStream_t s) {
   switch (epi) {
-    case MVIT_EPI_NONE: return launch<T, TO, TA, TB, MVIT_EPI_NONE>(p, s);
-    case MVIT_EPI_BIAS: return launch<T, TO, TA, TB, MVIT_EPI_BIAS>(p, s);
-    case MVIT_EPI_ACCUM: return launch<T, TO, TA, TB, MVIT_EPI_ACCUM>(p, s);
+    case MVIT_EPI_NONE: return launch_var<T, TO, TA, TB, MVIT_EPI_NONE>(var, p, s);
+    case MVIT_EPI_BIAS: return launch_var<T, TO, TA, TB, MVIT_EPI_BIAS>(var, p, s);
+    case MVIT_EPI_ACCUM: return launch_var<T, TO, TA, TB, MVIT_EPI_ACCUM>(var, p, s);
     default: break;
   }
   if constexpr (!TA && !TB) {
     // forward-only epilogues (both operands contraction-contiguous)
     switch (epi) {
-      case MVIT_EPI_BIAS_RES: return launch<T, TO, false, false, MVIT_EPI_BIAS_RES>(p, s);
-      case MVIT_EPI_BIAS_GELU: return launch<T, TO, false, false, MVIT_EPI_BIAS_GELU>(p, s);
-      case MVIT_EPI_SWIGLU: return launch<T, TO, false, false, MVIT_EPI_SWIGLU>(p, s);
+      case MVIT_EPI_BIAS_RES: return launch_var<T, TO, false, false, MVIT_EPI_BIAS_RES>(var, p, s);
+      case MVIT_EPI_BIAS_GELU: return launch_var<T, TO, false, false, MVIT_EPI_BIAS_GELU>(var, p, s);
+      case MVIT_EPI_SWIGLU: return launch_var<T, TO, false, false, MVIT_EPI_SWIGLU>(var, p, s);
       default: break;
     }
   }
   if constexpr (!TA && TB) {
     // data-gradient epilogues
     switch (epi) {
-      case MVIT_EPI_SWIGLU_BWD: return launch<T, TO, false, true, MVIT_EPI_SWIGLU_BWD>(p, s);
-      case MVIT_EPI_GELU_BWD: return launch<T, TO, false, true, MVIT_EPI_GELU_BWD>(p, s);
+      case MVIT_EPI_SWIGLU_BWD: return launch_var<T, TO, false, true, MVIT_EPI_SWIGLU_BWD>(var, p, s);
+      case MVIT_EPI_GELU_BWD: return launch_var<T, TO, false, true, MVIT_EPI_GELU_BWD>(var, p, s);
       default: break;
     }
   }
@@ -400,11 +544,15 @@ int dispatch_epi(int epi, const GemmParams& p, hipStream_t s) {
 }
 
 template <typename T, typename TO>
-int dispatch_trans(int ta, int tb, int epi, const GemmParams& p, hipStream_t s) {
-  if (!ta && !tb) return dispatch_epi<T, TO, false, false>(epi, p, s);
-  if (!ta && tb) return dispatch_epi<T, TO, false, true>(epi, p, s);
-  if (ta && tb) return dispatch_epi<T, TO, true, true>(epi, p, s);
+int dispatch_trans(int ta, int tb, int epi, int var, const GemmParams& p, hipStream_t s) {
+  if (!ta && !tb) return dispatch_epi<T, TO, false, false>(epi, var, p, s);
+  if (!ta && tb) return dispatch_epi<T, TO, false, true>(epi, var, p, s);
+  if (ta && tb) return dispatch_epi<T, TO, true, true>(epi, var, p, s);
   return mvit_set_error(MVIT_ERR_UNSUPPORTED, "gemm: trans_a=1, trans_b=0 is not built");
+}
+
+inline bool vec16(const void* ptr, int64_t ld, size_t esize) {
+  return ptr == nullptr || (mvit_aligned16(ptr) && (ld * (int64_t)esize) % 16 == 0);
 }
 
 }  // namespace
@@ -435,6 +583,9 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
   p.A = a->A; p.lda = a->lda; p.B = a->B; p.B2 = a->B2; p.ldb = a->ldb;
   p.bias = a->bias; p.bias2 = a->bias2; p.C = a->C; p.ldc = a->ldc;
   p.R = a->R; p.ldr = a->ldr; p.aux = a->aux; p.ldaux = a->ldaux; p.aux_off = a->aux_off;
+  const size_t es = a->dtype == MVIT_BF16 ? 2 : 4, eo = a->out_dtype == MVIT_BF16 ? 2 : 4;
+  p.vec_ok = vec16(a->C, a->ldc, eo) && vec16(a->R, a->ldr, es) && vec16(a->aux, a->ldaux, es) && vec16(a->bias, 0, es) &&
+             vec16(a->bias2, 0, es) && (a->aux_off * (int64_t)(es < eo ? es : eo)) % 16 == 0;
   const int n_per_block = (epi == MVIT_EPI_SWIGLU) ? BN / 2 : BN;
   const int64_t tm = (a->M + BM - 1) / BM, tn = (a->N + n_per_block - 1) / n_per_block;
   MVIT_REQUIRE(tm * tn < (1ll << 30), "gemm: too many tiles");
@@ -445,16 +596,17 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
     const int64_t chunk = ((a->K + a->split_k - 1) / a->split_k + bk - 1) / bk * bk;
     const int64_t slices = (a->K + chunk - 1) / chunk;  // never an empty slice
     MVIT_REQUIRE(epi == MVIT_EPI_NONE, "gemm: split_k is only available with EPI_NONE");
-    MVIT_REQUIRE(a->workspace && a->workspace_bytes >= (int64_t)sizeof(float) * slices * a->M * a->N,
-                 "gemm: split_k=%d needs a workspace of %lld bytes", a->split_k, (long long)(sizeof(float) * slices * a->M * a->N));
+    MVIT_REQUIRE(a->workspace && mvit_aligned16(a->workspace) && a->workspace_bytes >= (int64_t)sizeof(float) * slices * a->M * a->N,
+                 "gemm: split_k=%d needs a 16-byte aligned workspace of %lld bytes", a->split_k, (long long)(sizeof(float) * slices * a->M * a->N));
     MVIT_REQUIRE(tm * tn * slices < (1ll << 30), "gemm: too many tiles");
     if (slices > 1) { p.split_k = (int)slices; p.k_chunk = chunk; p.workspace = static_cast<float*>(a->workspace); }
   }
+  const int var = a->reserved == 1 ? 1 : 0;  // wave layout: 0 = 4 waves of 128x128, 1 = 8 waves of 128x64
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (a->dtype == MVIT_BF16) {
-    if (a->out_dtype == MVIT_BF16) return dispatch_trans<bf16_t, bf16_t>(a->trans_a, a->trans_b, epi, p, s);
-    return dispatch_trans<bf16_t, float>(a->trans_a, a->trans_b, epi, p, s);
+    if (a->out_dtype == MVIT_BF16) return dispatch_trans<bf16_t, bf16_t>(a->trans_a, a->trans_b, epi, var, p, s);
+    return dispatch_trans<bf16_t, float>(a->trans_a, a->trans_b, epi, var, p, s);
   }
   MVIT_REQUIRE(a->out_dtype == MVIT_F32, "gemm: fp32 operands need fp32 output");
-  return dispatch_trans<float, float>(a->trans_a, a->trans_b, epi, p, s);
+  return dispatch_trans<float, float>(a->trans_a, a->trans_b, epi, var, p, s);
 }

@@ -15,6 +15,10 @@ _DT = {torch.float32: F32, torch.bfloat16: BF16}
 N_PARTIAL = 256  # row-slice count of the two-stage column reductions
 
 
+import os as _os
+
+GEMM_VARIANT = int(_os.environ.get("MI355_VIT_GEMM_VARIANT", "1"))  # wave layout of the GEMM (0: 4 waves, 1: 8 waves)
+
 _trace = None  # optional list collecting (tag, info, start_event, end_event) per tagged launch
 
 
@@ -275,7 +279,7 @@ def gemm(
         raise ValueError(f"gemm: out {tuple(out.shape)} too small for M={M}, N={N}")
     args = GemmArgs()
     args.dtype, args.out_dtype = dt(a), dt(out)
-    args.trans_a, args.trans_b, args.epilogue = int(trans_a), int(trans_b), epilogue
+    args.trans_a, args.trans_b, args.epilogue, args.reserved = int(trans_a), int(trans_b), epilogue, GEMM_VARIANT
     args.M, args.N, args.K = M, N, K
     args.A, args.lda = a.data_ptr(), a.stride(0)
     args.B, args.ldb = b.data_ptr(), b.stride(0)
@@ -314,8 +318,8 @@ def gemm(
 
 
 def wgrad_split_k(out_rows: int, out_cols: int, k: int) -> int:
-    """K slices for a weight-gradient GEMM: few output tiles (256x128) but a long contraction (the tokens)."""
-    tiles = -(-out_rows // 256) * -(-out_cols // 128)
+    """K slices for a weight-gradient GEMM: few output tiles (256x256) but a long contraction (the tokens)."""
+    tiles = -(-out_rows // 256) * -(-out_cols // 256)
     want = max(1, min(16, round(768 / tiles)))
     return max(1, min(want, k // 512))
 
