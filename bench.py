@@ -68,14 +68,16 @@ def summarise_trace(records, cfg_kw, dtype):
     out = {}
     for tag, info, e0, e1 in records:
         ms = e0.elapsed_time(e1)
+        if tag.startswith("attn"):
+            tag += "_window" if info["max_seqlen"] <= 64 else "_full"
         ent = out.setdefault(tag, {"launches": 0, "ms": 0.0, "flops": 0.0, "bytes": 0.0})
         ent["launches"] += 1
         ent["ms"] += ms
         if tag.startswith("gemm"):
             ent["flops"] += 2.0 * info["M"] * unpad.get(info["N"], info["N"]) * unpad.get(info["K"], info["K"])
-        elif tag == "attn_fwd":
+        elif tag.startswith("attn_fwd"):
             ent["flops"] += 4.0 * seg_sq_sum(info["cu"].cpu()) * info["head_dim"] * info["nheads"]
-        elif tag == "attn_bwd":
+        elif tag.startswith("attn_bwd"):
             ent["flops"] += 10.0 * seg_sq_sum(info["cu"].cpu()) * info["head_dim"] * info["nheads"]
         elif tag == "rmsnorm_fwd":
             ent["bytes"] += 2.0 * info["rows"] * info["cols"] * info["esize"]
@@ -98,8 +100,10 @@ KERNEL_NAMES = {
     "gemm_nt_epi5": "gemm_kernel<.., TA=false, TB=true, EPI=SWIGLU_BWD>",
     "gemm_nt_epi6": "gemm_kernel<.., TA=false, TB=true, EPI=GELU_BWD>",
     "gemm_tt_epi0": "gemm_kernel<.., TA=true, TB=true, EPI=NONE>",
-    "attn_fwd": "attn_fwd_mfma<5, NWAVES>",
-    "attn_bwd": "attn_delta_kernel + attn_bwd_dkdv_mfma<5, NWAVES> + attn_bwd_dq_mfma<5, NWAVES>",
+    "attn_fwd_full": "attn_fwd_mfma<5, 4, 32, true>",
+    "attn_bwd_full": "attn_delta_kernel + attn_bwd_dkdv_mfma<5, 4> + attn_bwd_dq_mfma<5, 4>",
+    "attn_fwd_window": "attn_fwd_mfma<5, 1, 64, false>",
+    "attn_bwd_window": "attn_delta_kernel + attn_bwd_dkdv_mfma<5, 1> + attn_bwd_dq_mfma<5, 1>",
 }
 
 
@@ -211,8 +215,8 @@ def main() -> None:
         roofline = {"bound": "mfma", "kernel": KERNEL_NAMES.get(dom, dom), "launches_per_step": d["launches"],
                     "avg_launch_ms": d["ms"] / d["launches"], "achieved": ach, "peak": peak, "unit": "TFLOP/s",
                     "frac": ach / peak, "traffic": None}
-        a_ms = sum(summ[t]["ms"] for t in ("attn_fwd", "attn_bwd") if t in summ)
-        a_fl = sum(summ[t]["flops"] for t in ("attn_fwd", "attn_bwd") if t in summ)
+        a_ms = sum(v["ms"] for t, v in summ.items() if t.startswith("attn"))
+        a_fl = sum(v["flops"] for t, v in summ.items() if t.startswith("attn"))
         attn_util = a_fl / (a_ms * 1e-3) / 1e12 / peak if a_ms > 0 else None
         total_ms = sum(v["ms"] for v in summ.values())
         breakdown = {}

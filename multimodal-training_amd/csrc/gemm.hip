@@ -200,15 +200,17 @@ __device__ __forceinline__ float frag_f32(const float* lds, int row, int k) {
 }
 
 // Epilogue on 8 consecutive output columns n..n+7 of row m.  v: accumulators (gate half for SWIGLU), u: up half.
-template <typename T, typename TO, int EPI>
-__device__ __forceinline__ void emit8(const GemmParams& p, int64_t m, int64_t n, float* v, const float* u, bool vec) {
+// FULL: all 8 columns exist and every pointer allows 16-byte accesses (compile-time trip counts, vector memory
+// operations); otherwise a scalar path bounded by the matrix edge.
+template <typename T, typename TO, int EPI, bool FULL>
+__device__ __forceinline__ void emit8_impl(const GemmParams& p, int64_t m, int64_t n, float* v, const float* u) {
   TO* Cp = static_cast<TO*>(p.C);
   const T* Rp = static_cast<const T*>(p.R);
   T* auxp = static_cast<T*>(p.aux);
   const T* bias = static_cast<const T*>(p.bias);
   const T* bias2 = static_cast<const T*>(p.bias2);
-  const int cnt = (p.N - n) < 8 ? (int)(p.N - n) : 8;
-  vec = vec && cnt == 8;
+  const int cnt = FULL ? 8 : ((p.N - n) < 8 ? (int)(p.N - n) : 8);
+  constexpr bool vec = FULL;
 
   if constexpr (EPI == MVIT_EPI_BIAS || EPI == MVIT_EPI_BIAS_RES || EPI == MVIT_EPI_BIAS_GELU || EPI == MVIT_EPI_SWIGLU) {
     if (bias) {
@@ -312,6 +314,12 @@ __device__ __forceinline__ void emit8(const GemmParams& p, int64_t m, int64_t n,
   if (vec) store8(c_out, v);
   else
     for (int e = 0; e < cnt; ++e) c_out[e] = from_f32<TO>(v[e]);
+}
+
+template <typename T, typename TO, int EPI>
+__device__ __forceinline__ void emit8(const GemmParams& p, int64_t m, int64_t n, float* v, const float* u, bool vec) {
+  if (vec && n + 8 <= p.N) emit8_impl<T, TO, EPI, true>(p, m, n, v, u);
+  else emit8_impl<T, TO, EPI, false>(p, m, n, v, u);
 }
 
 template <typename T, typename TO, bool TA, bool TB, int EPI, int VAR>
