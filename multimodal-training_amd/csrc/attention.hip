@@ -375,10 +375,10 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const T* __restrict__ o
 // ================================================================================================
 // dK, dV.  Block = 64*NWAVES keys of one (segment, head); 32 queries per iteration, Q / dO tiles (and the
 // rows' lse, delta) double buffered in LDS with the next tile's loads in flight during the MFMAs.
-template <int ND, int NWAVES>
+template <int ND, int NWAVES, int RB>
 __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnParams p) {
   using G = Geo<ND>;
-  constexpr int HD = G::HD, BQ = 32, NT = 64 * NWAVES;
+  constexpr int HD = G::HD, BQ = 32, NT = 64 * NWAVES, SPAN = 16 * RB * NWAVES;  // RB 16-row blocks per wave
   __shared__ __attribute__((aligned(16))) bf16_t lds_q[2][BQ * G::PK];
   __shared__ __attribute__((aligned(16))) bf16_t lds_do[2][BQ * G::PK];
   __shared__ __attribute__((aligned(16))) float lds_lse[2][BQ];
@@ -386,10 +386,10 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
 
   const int seg = blockIdx.y, h = blockIdx.z;
   const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
-  const int blk_k0 = blockIdx.x * NT;
+  const int blk_k0 = blockIdx.x * SPAN;
   if (blk_k0 >= L) return;
   const int l = threadIdx.x & 63, wv = threadIdx.x >> 6, g = l >> 4, r = l & 15;
-  const int key0 = blk_k0 + wv * 64;
+  const int key0 = blk_k0 + wv * 16 * RB;
 
   const bf16_t* Q = static_cast<const bf16_t*>(p.q) + (int64_t)s0 * p.q_stride + (int64_t)h * HD;
   const bf16_t* K = static_cast<const bf16_t*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD;
@@ -398,16 +398,16 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
   const float* LSE = p.lse + (int64_t)h * p.total + s0;
   const float* DELTA = p.delta + (int64_t)h * p.total + s0;
 
-  RowFrag<ND> kf[4], vf[4];
+  RowFrag<ND> kf[RB], vf[RB];
 #pragma unroll
-  for (int kb = 0; kb < 4; ++kb) {
+  for (int kb = 0; kb < RB; ++kb) {
     const int ki = key0 + kb * 16 + r;
     load_rowfrag_global<ND>(kf[kb], K + (int64_t)ki * p.k_stride, ki < L, g);
     load_rowfrag_global<ND>(vf[kb], V + (int64_t)ki * p.v_stride, ki < L, g);
   }
-  f32x4 dk[4][ND], dv[4][ND];
+  f32x4 dk[RB][ND], dv[RB][ND];
 #pragma unroll
-  for (int kb = 0; kb < 4; ++kb)
+  for (int kb = 0; kb < RB; ++kb)
 #pragma unroll
     for (int dt = 0; dt < ND; ++dt) {
       dk[kb][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -469,7 +469,7 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
       dt_[d] = tr_pair(tdo + off, tdo + off + 16 * G::PK);
     }
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
+    for (int kb = 0; kb < RB; ++kb) {
       f32x4 pv[2], ds[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
@@ -502,7 +502,7 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
   bf16_t* DK = static_cast<bf16_t*>(p.dk) + (int64_t)s0 * p.dk_stride + (int64_t)h * HD;
   bf16_t* DV = static_cast<bf16_t*>(p.dv) + (int64_t)s0 * p.dv_stride + (int64_t)h * HD;
 #pragma unroll
-  for (int kb = 0; kb < 4; ++kb) {
+  for (int kb = 0; kb < RB; ++kb) {
     const int ki = key0 + kb * 16 + r;
     if (ki < L) {
 #pragma unroll
@@ -522,19 +522,19 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
 
 // ================================================================================================
 // dQ.  Block = 64*NWAVES queries of one (segment, head); 32 keys per iteration, K / V tiles double buffered.
-template <int ND, int NWAVES>
+template <int ND, int NWAVES, int RB>
 __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams p) {
   using G = Geo<ND>;
-  constexpr int HD = G::HD, BK = 32, NT = 64 * NWAVES;
+  constexpr int HD = G::HD, BK = 32, NT = 64 * NWAVES, SPAN = 16 * RB * NWAVES;  // RB 16-row blocks per wave
   __shared__ __attribute__((aligned(16))) bf16_t lds_k[2][BK * G::PK];
   __shared__ __attribute__((aligned(16))) bf16_t lds_v[2][BK * G::PK];
 
   const int seg = blockIdx.y, h = blockIdx.z;
   const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
-  const int blk_q0 = blockIdx.x * NT;
+  const int blk_q0 = blockIdx.x * SPAN;
   if (blk_q0 >= L) return;
   const int l = threadIdx.x & 63, wv = threadIdx.x >> 6, g = l >> 4, r = l & 15;
-  const int q0 = blk_q0 + wv * 64;
+  const int q0 = blk_q0 + wv * 16 * RB;
 
   const bf16_t* Q = static_cast<const bf16_t*>(p.q) + (int64_t)s0 * p.q_stride + (int64_t)h * HD;
   const bf16_t* K = static_cast<const bf16_t*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD;
@@ -543,10 +543,10 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams
   const float* LSE = p.lse + (int64_t)h * p.total + s0;
   const float* DELTA = p.delta + (int64_t)h * p.total + s0;
 
-  RowFrag<ND> qf[4], dof[4];
-  float neg_lse2[4], dl[4];
+  RowFrag<ND> qf[RB], dof[RB];
+  float neg_lse2[RB], dl[RB];
 #pragma unroll
-  for (int qb = 0; qb < 4; ++qb) {
+  for (int qb = 0; qb < RB; ++qb) {
     const int qi = q0 + qb * 16 + r;
     const bool ok = qi < L;
     load_rowfrag_global<ND>(qf[qb], Q + (int64_t)qi * p.q_stride, ok, g);
@@ -554,9 +554,9 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams
     neg_lse2[qb] = ok ? -LSE[qi] * LOG2E : -INFINITY;
     dl[qb] = ok ? DELTA[qi] : 0.f;
   }
-  f32x4 dq[4][ND];
+  f32x4 dq[RB][ND];
 #pragma unroll
-  for (int qb = 0; qb < 4; ++qb)
+  for (int qb = 0; qb < RB; ++qb)
 #pragma unroll
     for (int d = 0; d < ND; ++d) dq[qb][d] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float c = p.scale * LOG2E;
@@ -595,7 +595,7 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams
       kt[d] = tr_pair(tk + off, tk + off + 16 * G::PK);
     }
 #pragma unroll
-    for (int qb = 0; qb < 4; ++qb) {
+    for (int qb = 0; qb < RB; ++qb) {
       f32x4 ds[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
@@ -628,7 +628,7 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams
 
   bf16_t* DQ = static_cast<bf16_t*>(p.dq) + (int64_t)s0 * p.dq_stride + (int64_t)h * HD;
 #pragma unroll
-  for (int qb = 0; qb < 4; ++qb) {
+  for (int qb = 0; qb < RB; ++qb) {
     const int qi = q0 + qb * 16 + r;
     if (qi < L) {
 #pragma unroll
@@ -839,17 +839,19 @@ int launch_fwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
 }
 template <int ND>
 int launch_bwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t s) {
-  const int nw = pick_waves(max_seqlen);
-  dim3 grid((unsigned)((max_seqlen + 64 * nw - 1) / (64 * nw)), (unsigned)n_seg, (unsigned)p.nheads);
-  if (nw == 1) {
-    hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 1>), grid, 64, 0, s, p);
-    hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 1>), grid, 64, 0, s, p);
-  } else if (nw == 2) {
-    hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 2>), grid, 128, 0, s, p);
-    hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 2>), grid, 128, 0, s, p);
+  // short segments (windows): one wave owns a whole 64-row block; long ones: 8 waves x 32 rows (2 waves per SIMD)
+  if (max_seqlen <= 64) {
+    dim3 grid(1, (unsigned)n_seg, (unsigned)p.nheads);
+    hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 1, 4>), grid, 64, 0, s, p);
+    hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 1, 4>), grid, 64, 0, s, p);
+  } else if (max_seqlen <= 128) {
+    dim3 grid(1, (unsigned)n_seg, (unsigned)p.nheads);
+    hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 2, 4>), grid, 128, 0, s, p);
+    hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 2, 4>), grid, 128, 0, s, p);
   } else {
-    hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 4>), grid, 256, 0, s, p);
-    hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 4>), grid, 256, 0, s, p);
+    dim3 grid((unsigned)((max_seqlen + 255) / 256), (unsigned)n_seg, (unsigned)p.nheads);
+    hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 8, 2>), grid, 512, 0, s, p);
+    hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 8, 2>), grid, 512, 0, s, p);
   }
   MVIT_CHECK_LAUNCH("attn_bwd");
   return MVIT_OK;

@@ -12,7 +12,7 @@ from . import _lib
 from ._lib import BF16, F32, GemmArgs
 
 _DT = {torch.float32: F32, torch.bfloat16: BF16}
-N_PARTIAL = 256  # row-slice count of the two-stage column reductions
+N_PARTIAL = 1024  # work-groups (= partial rows) of the RMSNorm backward: 4 per CU keep enough loads in flight
 
 
 import os as _os
