@@ -17,7 +17,6 @@
 
 namespace {
 
-constexpr int BM = 256, BN = 256;
 
 struct GemmParams {
   int64_t M, N, K;
@@ -60,12 +59,16 @@ struct Cfg<float> {
 template <int VAR>
 struct Waves;
 template <>
-struct Waves<0> {
-  static constexpr int WM = 128, WN = 128, NTHREADS = 256;
+struct Waves<0> {  // 256x256 tile, 4 waves of 128x128, double-buffered LDS, one work-group per CU
+  static constexpr int BM = 256, BN = 256, WM = 128, WN = 128, NTHREADS = 256, STAGES = 2, MIN_WAVES = 1;
 };
 template <>
-struct Waves<1> {
-  static constexpr int WM = 128, WN = 64, NTHREADS = 512;
+struct Waves<1> {  // 256x256 tile, 8 waves of 128x64, double-buffered LDS, one work-group per CU
+  static constexpr int BM = 256, BN = 256, WM = 128, WN = 64, NTHREADS = 512, STAGES = 2, MIN_WAVES = 2;
+};
+template <>
+struct Waves<2> {  // 256x128 tile, 4 waves of 128x64, single LDS buffer: two independent work-groups per CU
+  static constexpr int BM = 256, BN = 128, WM = 128, WN = 64, NTHREADS = 256, STAGES = 1, MIN_WAVES = 2;
 };
 
 __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.f + erff(z * 0.70710678118654752440f)); }
@@ -103,7 +106,11 @@ __device__ __forceinline__ void store8(float* p, const float* v) {
 
 // Stage one operand tile (ROWS rows of the output dimension x BK of the contraction) global -> registers -> LDS.
 // TR = false: memory is [row][k];  TR = true: memory is [k][row].
-template <typename T, int ROWS, bool TR, int NTHREADS, int WN>
+// A thread's chunks are a fixed distance apart (NTHREADS/8 rows, or NTHREADS/(ROWS/V) k-rows when TR), so one
+// pointer, one remaining-K counter and a row mask describe the whole K loop.  Loads are unconditional (masked
+// chunks read the operand's first element) and zeroed, if need be, when written to LDS.
+// DUAL (SWIGLU's B operand): rows alternate between two matrices, so every chunk keeps its own pointer.
+template <typename T, int ROWS, bool TR, int NTHREADS, int WN, bool DUAL>
 struct TileLoader {
   using C = Cfg<T>;
   static constexpr int V = C::VEC;
@@ -111,48 +118,70 @@ struct TileLoader {
   static constexpr int CHUNKS = ROWS * C::BK / V;  // 16-byte chunks per tile
   static constexpr int PER_THREAD = CHUNKS / NTHREADS;
   static constexpr int LDS_ELEMS = TR ? C::BK * (ROWS + C::PAD_T) : ROWS * C::PITCH_K;
+  static constexpr int ROW_STEP = TR ? 0 : NTHREADS / (C::BK / V);  // tile rows between consecutive chunks
+  static constexpr int K_STEP = TR ? NTHREADS / (ROWS / V) : 0;     // k between consecutive chunks
   vec_t regs[PER_THREAD];
+  const T* ptr[DUAL ? PER_THREAD : 1];
+  const T* safe;      // always-valid address for masked chunks
+  int64_t chunk_step; // elements between consecutive chunks of this thread
+  int64_t step;       // pointer advance per K tile
+  int k_left;         // K elements left from chunk 0's position (<= 0: exhausted)
+  unsigned row_mask;  // bit i: chunk i lies on a valid row
 
-  // dual: SWIGLU packs two weight matrices into one B tile so that a wave's first N sub-tiles are gate columns and
-  // its last ones the up columns with the same indices: tile row r = wn*WN + half*(WN/2) + j -> matrix `half`,
-  // row row0 + wn*(WN/2) + j.
-  __device__ __forceinline__ void load(const T* __restrict__ base, const T* __restrict__ base2, int64_t ld,
-                                       int64_t row0, int64_t row_limit, int64_t k0, int64_t k_end, bool dual) {
+  __device__ __forceinline__ void init(const T* __restrict__ base, const T* __restrict__ base2, int64_t ld,
+                                       int64_t row0, int64_t row_limit, int64_t k_begin, int64_t k_end) {
+    step = TR ? (int64_t)C::BK * ld : (int64_t)C::BK;
+    chunk_step = TR ? (int64_t)K_STEP * ld : (int64_t)ROW_STEP * ld;
+    safe = base;
+    row_mask = 0;
+    const int c0 = threadIdx.x;
+    const int kk0 = TR ? c0 / (ROWS / V) : (c0 % (C::BK / V)) * V;
+    const int64_t left = k_end - (k_begin + kk0);
+    k_left = (int)(left > (1 << 30) ? (1 << 30) : left);
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
       const int c = threadIdx.x + NTHREADS * i;
-      int r, kk;
-      if (!TR) {
-        r = c / (C::BK / V);
-        kk = (c % (C::BK / V)) * V;
-      } else {
-        kk = c / (ROWS / V);
-        r = (c % (ROWS / V)) * V;
-      }
+      const int r = TR ? (c % (ROWS / V)) * V : c / (C::BK / V);
+      const int kk = TR ? c / (ROWS / V) : (c % (C::BK / V)) * V;
       const T* src = base;
-      int64_t grow;
-      if (dual) {
+      int64_t grow = row0 + r;
+      if (DUAL) {  // tile row r = wn*WN + half*(WN/2) + j -> matrix `half`, row row0 + wn*(WN/2) + j
         const int wn = r / WN, w = r % WN, half = w / (WN / 2), j = w % (WN / 2);
         grow = row0 + wn * (WN / 2) + j;
         if (half) src = base2;
-      } else {
-        grow = row0 + r;
       }
-      const int64_t gk = k0 + kk;
-      vec_t v;
+      const bool row_ok = grow < row_limit;
+      if (row_ok) row_mask |= 1u << i;
+      const int64_t gk = k_begin + kk;
+      const T* q = row_ok ? (TR ? src + gk * ld + grow : src + grow * ld + gk) : src;
+      if (DUAL) ptr[i] = q;
+      else if (i == 0) ptr[0] = TR ? src + gk * ld + grow : src + grow * ld + gk;  // may lie past the edge: never dereferenced then
+    }
+  }
+  __device__ __forceinline__ bool live(int i, int kl) const { return ((row_mask >> i) & 1u) && (kl - i * K_STEP > 0); }
+  __device__ __forceinline__ void load() {
 #pragma unroll
-      for (int j = 0; j < V; ++j) v[j] = from_f32<T>(0.f);
-      if (!TR) {
-        if (grow < row_limit && gk < k_end) v = *reinterpret_cast<const vec_t*>(src + grow * ld + gk);
-      } else {
-        if (grow < row_limit && gk < k_end) v = *reinterpret_cast<const vec_t*>(src + gk * ld + grow);
-      }
-      regs[i] = v;
+    for (int i = 0; i < PER_THREAD; ++i) {
+      const bool ok = live(i, k_left);
+      const T* q = DUAL ? ptr[i] : ptr[0] + i * chunk_step;
+      regs[i] = *reinterpret_cast<const vec_t*>(ok ? q : safe);
+    }
+    k_left -= C::BK;
+    if (DUAL) {
+#pragma unroll
+      for (int i = 0; i < PER_THREAD; ++i) ptr[i] += step;
+    } else {
+      ptr[0] += step;
     }
   }
   __device__ __forceinline__ void store(T* lds) const {
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
+      vec_t v = regs[i];
+      if (!live(i, k_left + C::BK)) {  // this chunk was outside the matrix / K range when it was loaded
+#pragma unroll
+        for (int j = 0; j < V; ++j) v[j] = from_f32<T>(0.f);
+      }
       const int c = threadIdx.x + NTHREADS * i;
       int off;
       if (!TR) {
@@ -162,7 +191,7 @@ struct TileLoader {
         const int kk = c / (ROWS / V), r = (c % (ROWS / V)) * V;
         off = kk * (ROWS + C::PAD_T) + r;
       }
-      *reinterpret_cast<vec_t*>(lds + off) = regs[i];
+      *reinterpret_cast<vec_t*>(lds + off) = v;
     }
   }
 };
@@ -322,104 +351,15 @@ __device__ __forceinline__ void emit8(const GemmParams& p, int64_t m, int64_t n,
   else emit8_impl<T, TO, EPI, false>(p, m, n, v, u);
 }
 
-template <typename T, typename TO, bool TA, bool TB, int EPI, int VAR>
-__global__ __launch_bounds__(Waves<VAR>::NTHREADS) void gemm_kernel(const GemmParams p) {
-  using C = Cfg<T>;
-  using W = Waves<VAR>;
-  constexpr int BK = C::BK, WM = W::WM, WN = W::WN, NTHREADS = W::NTHREADS;
-  constexpr int MT = WM / 32, NT = WN / 32, WGN = BN / WN;  // waves along N
-  using LoaderA = TileLoader<T, BM, TA, NTHREADS, WN>;
-  using LoaderB = TileLoader<T, BN, TB, NTHREADS, WN>;
-  constexpr int STAGE_ELEMS = LoaderA::LDS_ELEMS + LoaderB::LDS_ELEMS;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  T* lds = reinterpret_cast<T*>(smem_raw);
-
-  // XCD-aware tile order: hardware deals consecutive work-group ids round-robin to the 8 XCDs; give each
-  // XCD a contiguous range of tiles (N fastest) so that its L2 sees one A panel at a time.
-  // With split-K the slices are the slowest index: all tiles of one K slice share the same rows of A and B.
-  const int tiles = p.tiles_m * p.tiles_n;
-  const int total = tiles * p.split_k;
-  const int per_xcd = (total + 7) / 8;
-  const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (work >= total) return;
-  const int slice = work / tiles, tile = work % tiles;
-  const int tm = tile / p.tiles_n, tn = tile % p.tiles_n;
-  const int64_t k_begin = (int64_t)slice * p.k_chunk;
-  const int64_t k_end = p.split_k > 1 ? (k_begin + p.k_chunk < p.K ? k_begin + p.k_chunk : p.K) : p.K;
+// Epilogue shared by every main loop.  acc[a][b][4*j+i] is C[m0 + wm*WM + a*32 + 8*j + 4*(l/32) + i][wave column
+// b*32 + l%32].  Pass a: every wave parks its a-th 32-row sub-tile in LDS (fp32, [(BM/WM)*32 rows][BN + 8]), then
+// the block walks the pass in 8-column groups.  The caller guarantees that no wave still reads operands from LDS.
+template <typename T, typename TO, int EPI, int BM, int BN, int WM, int WN, int NTHREADS>
+__device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[WM / 32][WN / 32], unsigned char* smem_raw,
+                                             int64_t m0, int64_t n0, int wm, int wn, int slice) {
+  constexpr int MT = WM / 32, NT = WN / 32;
   constexpr bool DUAL = (EPI == MVIT_EPI_SWIGLU);
-  constexpr int N_PER_BLOCK = DUAL ? BN / 2 : BN;
-  const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * N_PER_BLOCK;
-
-  const int l = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int wm = wv / WGN, wn = wv % WGN;
-
-  f32x16 acc[MT][NT];
-#pragma unroll
-  for (int a = 0; a < MT; ++a)
-#pragma unroll
-    for (int b = 0; b < NT; ++b)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
-
-  LoaderA la;
-  LoaderB lb;
-  const T* A = static_cast<const T*>(p.A);
-  const T* B = static_cast<const T*>(p.B);
-  const T* B2 = static_cast<const T*>(p.B2);
-  la.load(A, nullptr, p.lda, m0, p.M, k_begin, k_end, false);
-  lb.load(B, B2, p.ldb, n0, p.N, k_begin, k_end, DUAL);
-  la.store(lds);
-  lb.store(lds + LoaderA::LDS_ELEMS);
-  __syncthreads();
-
-  int buf = 0;
-  for (int64_t k0 = k_begin; k0 < k_end; k0 += BK) {
-    const bool has_next = k0 + BK < k_end;
-    if (has_next) {
-      la.load(A, nullptr, p.lda, m0, p.M, k0 + BK, k_end, false);
-      lb.load(B, B2, p.ldb, n0, p.N, k0 + BK, k_end, DUAL);
-    }
-    const T* lds_a = lds + buf * STAGE_ELEMS;
-    const T* lds_b = lds_a + LoaderA::LDS_ELEMS;
-    if constexpr (sizeof(T) == 2) {
-#pragma unroll
-      for (int ks = 0; ks < BK; ks += 16) {
-        bf16x8 fa[MT], fb[NT];
-#pragma unroll
-        for (int a = 0; a < MT; ++a) fa[a] = frag_bf16<TA, BM>(reinterpret_cast<const bf16_t*>(lds_a), wm * WM + a * 32, ks);
-#pragma unroll
-        for (int b = 0; b < NT; ++b) fb[b] = frag_bf16<TB, BN>(reinterpret_cast<const bf16_t*>(lds_b), wn * WN + b * 32, ks);
-#pragma unroll
-        for (int a = 0; a < MT; ++a)
-#pragma unroll
-          for (int b = 0; b < NT; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[a], fb[b], acc[a][b], 0, 0, 0);
-      }
-    } else {
-#pragma unroll
-      for (int ks = 0; ks < BK; ks += 2) {
-        float fa[MT], fb[NT];
-#pragma unroll
-        for (int a = 0; a < MT; ++a) fa[a] = frag_f32<TA, BM>(reinterpret_cast<const float*>(lds_a), wm * WM + a * 32, ks);
-#pragma unroll
-        for (int b = 0; b < NT; ++b) fb[b] = frag_f32<TB, BN>(reinterpret_cast<const float*>(lds_b), wn * WN + b * 32, ks);
-#pragma unroll
-        for (int a = 0; a < MT; ++a)
-#pragma unroll
-          for (int b = 0; b < NT; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a], fb[b], acc[a][b], 0, 0, 0);
-      }
-    }
-    if (has_next) {
-      T* nxt = lds + (buf ^ 1) * STAGE_ELEMS;
-      la.store(nxt);
-      lb.store(nxt + LoaderA::LDS_ELEMS);
-    }
-    __syncthreads();
-    buf ^= 1;
-  }
-
-  // ---- epilogue.  acc[a][b][4*j+i] is C[m0 + wm*WM + a*32 + 8*j + 4*(l/32) + i][wave column b*32 + l%32].
-  // Pass a: every wave parks its a-th 32-row sub-tile in LDS (fp32, [ (BM/WM)*32 rows ][ BN + 8 ]), then the block
-  // walks the pass in 8-column groups.
+  const int l = threadIdx.x & 63;
   constexpr int SP = BN + 8;
   constexpr int PASS_ROWS = (BM / WM) * 32;
   constexpr int NCOLS = DUAL ? BN / 2 : BN;
@@ -476,6 +416,347 @@ __global__ __launch_bounds__(Waves<VAR>::NTHREADS) void gemm_kernel(const GemmPa
   }
 }
 
+template <typename T, typename TO, bool TA, bool TB, int EPI, int VAR>
+__global__ __launch_bounds__(Waves<VAR>::NTHREADS, Waves<VAR>::MIN_WAVES) void gemm_kernel(const GemmParams p) {
+  using C = Cfg<T>;
+  using W = Waves<VAR>;
+  constexpr int BK = C::BK, BM = W::BM, BN = W::BN, WM = W::WM, WN = W::WN, NTHREADS = W::NTHREADS, STAGES = W::STAGES;
+  constexpr int MT = WM / 32, NT = WN / 32, WGN = BN / WN;  // waves along N
+  constexpr bool DUAL = (EPI == MVIT_EPI_SWIGLU);
+  using LoaderA = TileLoader<T, BM, TA, NTHREADS, WN, false>;
+  using LoaderB = TileLoader<T, BN, TB, NTHREADS, WN, DUAL>;
+  constexpr int STAGE_ELEMS = LoaderA::LDS_ELEMS + LoaderB::LDS_ELEMS;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T* lds = reinterpret_cast<T*>(smem_raw);
+
+  // XCD-aware tile order: hardware deals consecutive work-group ids round-robin to the 8 XCDs; give each
+  // XCD a contiguous range of tiles (N fastest) so that its L2 sees one A panel at a time.
+  // With split-K the slices are the slowest index: all tiles of one K slice share the same rows of A and B.
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int total = tiles * p.split_k;
+  const int per_xcd = (total + 7) / 8;
+  const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (work >= total) return;
+  const int slice = work / tiles, tile = work % tiles;
+  const int tm = tile / p.tiles_n, tn = tile % p.tiles_n;
+  const int64_t k_begin = (int64_t)slice * p.k_chunk;
+  const int64_t k_end = p.split_k > 1 ? (k_begin + p.k_chunk < p.K ? k_begin + p.k_chunk : p.K) : p.K;
+  constexpr int N_PER_BLOCK = DUAL ? BN / 2 : BN;
+  const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * N_PER_BLOCK;
+
+  const int l = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int wm = wv / WGN, wn = wv % WGN;
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int a = 0; a < MT; ++a)
+#pragma unroll
+    for (int b = 0; b < NT; ++b)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
+
+  LoaderA la;
+  LoaderB lb;
+  const T* A = static_cast<const T*>(p.A);
+  const T* B = static_cast<const T*>(p.B);
+  const T* B2 = static_cast<const T*>(p.B2);
+  la.init(A, nullptr, p.lda, m0, p.M, k_begin, k_end);
+  lb.init(B, B2, p.ldb, n0, p.N, k_begin, k_end);
+  la.load();
+  lb.load();
+  if (STAGES == 2) {
+    la.store(lds);
+    lb.store(lds + LoaderA::LDS_ELEMS);
+    __syncthreads();
+  }
+
+  int buf = 0;
+  for (int64_t k0 = k_begin; k0 < k_end; k0 += BK) {
+    const bool has_next = k0 + BK < k_end;
+    if (STAGES == 1) {
+      if (k0 > k_begin) __syncthreads();  // the previous tile has been consumed by every wave
+      la.store(lds);
+      lb.store(lds + LoaderA::LDS_ELEMS);
+      __syncthreads();
+    }
+    if (has_next) {
+      la.load();
+      lb.load();
+    }
+    const T* lds_a = lds + buf * STAGE_ELEMS;
+    const T* lds_b = lds_a + LoaderA::LDS_ELEMS;
+    if constexpr (sizeof(T) == 2) {
+      // operand fragments are fetched one 16-wide step ahead of the MFMAs that consume them
+      const bf16_t* la_ = reinterpret_cast<const bf16_t*>(lds_a);
+      const bf16_t* lb_ = reinterpret_cast<const bf16_t*>(lds_b);
+      bf16x8 fa[2][MT], fb[2][NT];
+#pragma unroll
+      for (int a = 0; a < MT; ++a) fa[0][a] = frag_bf16<TA, BM>(la_, wm * WM + a * 32, 0);
+#pragma unroll
+      for (int b = 0; b < NT; ++b) fb[0][b] = frag_bf16<TB, BN>(lb_, wn * WN + b * 32, 0);
+#pragma unroll
+      for (int s4 = 0; s4 < BK / 16; ++s4) {
+        const int cur = s4 & 1, nxt = cur ^ 1;
+        if (s4 + 1 < BK / 16) {
+#pragma unroll
+          for (int a = 0; a < MT; ++a) fa[nxt][a] = frag_bf16<TA, BM>(la_, wm * WM + a * 32, (s4 + 1) * 16);
+#pragma unroll
+          for (int b = 0; b < NT; ++b) fb[nxt][b] = frag_bf16<TB, BN>(lb_, wn * WN + b * 32, (s4 + 1) * 16);
+        }
+        __builtin_amdgcn_sched_barrier(0);  // keep the fetches of step s4+1 ahead of the MFMAs of step s4
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+          for (int b = 0; b < NT; ++b)
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][a], fb[cur][b], acc[a][b], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < BK; ks += 2) {
+        float fa[MT], fb[NT];
+#pragma unroll
+        for (int a = 0; a < MT; ++a) fa[a] = frag_f32<TA, BM>(reinterpret_cast<const float*>(lds_a), wm * WM + a * 32, ks);
+#pragma unroll
+        for (int b = 0; b < NT; ++b) fb[b] = frag_f32<TB, BN>(reinterpret_cast<const float*>(lds_b), wn * WN + b * 32, ks);
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+          for (int b = 0; b < NT; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a], fb[b], acc[a][b], 0, 0, 0);
+      }
+    }
+    if (STAGES == 2) {
+      if (has_next) {
+        T* nxt = lds + (buf ^ 1) * STAGE_ELEMS;
+        la.store(nxt);
+        lb.store(nxt + LoaderA::LDS_ELEMS);
+      }
+      __syncthreads();
+      buf ^= 1;
+    }
+  }
+  if (STAGES == 1) __syncthreads();  // operands fully consumed before LDS is reused for the epilogue
+
+  run_epilogue<T, TO, EPI, BM, BN, WM, WN, NTHREADS>(p, acc, smem_raw, m0, n0, wm, wn, slice);
+}
+
+// ---- bf16 main loop with direct global -> LDS loads (no staging registers) ----------------------------------
+// 256x256 tile, 8 waves of 128x64, BK = 32, NSTAGE LDS stages of 16 KiB per operand.  global_load_lds_dwordx4 moves
+// 16 bytes per lane straight into LDS at M0 + 16*lane, so one wave instruction fills 1 KiB of contiguous LDS and
+// NSTAGE-1 K tiles are in flight while one is consumed; addresses are a per-lane 32-bit offset (constant over the
+// K loop) plus a wave-uniform 64-bit base that a scalar add advances.  Because the LDS image of one instruction
+// is contiguous, bank conflicts are avoided by permuting which global chunk a lane fetches:
+//   [row][k] operands: 64-byte rows of 4 chunks, chunk c of row r lives in slot c ^ ((r >> 2) & 3);
+//   [k][row] operands: 512-byte k-rows of 32 chunks, chunk c of k-row k lives in slot c ^ ((k & 3) << 2).
+// Rows past the matrix edge are clamped to valid rows (they only feed outputs that are never stored).  A partial
+// last K tile (K not a multiple of 32) is loaded through registers with zeros past the end of K.
+// The compiler does not see these loads: s_waitcnt vmcnt is placed by hand (loads return in order).
+struct DL {
+  static constexpr int BM = 256, BN = 256, BK = 32, WM = 128, WN = 64, NTHREADS = 512, NSTAGE = 4;
+  static constexpr int TILE_BYTES = 256 * BK * 2;
+};
+
+__device__ __forceinline__ void dl_load(unsigned lds_addr, unsigned voff, const char* base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+template <bool TR, bool DUAL>
+struct DlOperand {
+  unsigned voff[2];     // byte offset of this lane's two 16-byte chunks from base[i]
+  const char* base[2];  // wave-uniform, advanced by `step` every K tile (DUAL: the two matrices)
+  int64_t step;
+
+  __device__ __forceinline__ void init(const bf16_t* X, const bf16_t* X2, int64_t ld, int64_t row0, int64_t limit,
+                                       int64_t k_begin, int wv) {
+    const int l = threadIdx.x & 63;
+    step = TR ? 2 * DL::BK * ld : 2 * DL::BK;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int q = wv * 2 + i;  // which 1 KiB of the stage this instruction fills
+      if (!TR) {
+        const int r = q * 16 + (l >> 2), c = (l & 3) ^ ((r >> 2) & 3);
+        int64_t grow = row0 + r;
+        const bf16_t* src = X;
+        if (DUAL) {  // tile row r = wn*WN + half*(WN/2) + j  ->  matrix `half` (uniform per wave), row row0 + wn*(WN/2) + j
+          grow = row0 + (r / DL::WN) * (DL::WN / 2) + (r % (DL::WN / 2));
+          if (wv & 1) src = X2;
+        }
+        if (grow >= limit) grow = limit - 1;
+        voff[i] = (unsigned)(((grow - row0) * ld + c * 8) * 2);
+        base[i] = reinterpret_cast<const char*>(src + row0 * ld + k_begin);
+      } else {
+        const int kr = 2 * q + (l >> 5);
+        int ch = (l & 31) ^ ((kr & 3) << 2);
+        if (row0 + ch * 8 >= limit) ch = 0;
+        voff[i] = (unsigned)((kr * ld + ch * 8) * 2);
+        base[i] = reinterpret_cast<const char*>(X + k_begin * ld + row0);
+      }
+    }
+  }
+  // lds_addr: LDS byte address of this wave's 2 KiB slice of the operand's stage
+  __device__ __forceinline__ void issue(unsigned lds_addr) {
+    dl_load(lds_addr, voff[0], base[0]);
+    dl_load(lds_addr + 1024, voff[1], base[1]);
+    base[0] += step;
+    base[1] += step;
+  }
+  __device__ __forceinline__ void issue_tail(unsigned char* lds_slice, int k_rem, int wv) {
+    const int l = threadIdx.x & 63;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int q = wv * 2 + i;
+      int k;  // first contraction index of the chunk
+      if (!TR) {
+        const int r = q * 16 + (l >> 2);
+        k = ((l & 3) ^ ((r >> 2) & 3)) * 8;
+      } else {
+        k = 2 * q + (l >> 5);
+      }
+      bf16x8 v;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = from_f32<bf16_t>(0.f);
+      if (k < k_rem) v = *reinterpret_cast<const bf16x8*>(base[i] + voff[i]);
+      *reinterpret_cast<bf16x8*>(lds_slice + i * 1024 + l * 16) = v;
+    }
+  }
+};
+
+// MFMA operand fetch for the DL layout: sub-tile `a` (32 rows) of the wave, 16-wide contraction step ks, stage s.
+template <bool TR, int NSUB>
+struct DlFrag {
+  unsigned off[TR ? NSUB : 2];
+  __device__ __forceinline__ void init(int rowbase, unsigned region) {
+    const int l = threadIdx.x & 63;
+    if (!TR) {
+      const int x = ((l & 31) >> 2) & 3;
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) off[ks] = region + (rowbase + (l & 31)) * 64 + (((ks * 2 + (l >> 5)) ^ x) << 4);
+    } else {
+      // lane i of 16-lane group G fetches 4 rows of k-row 8*(G/2) + i/4 at row 16*(G%2) + 4*(i%4); the transposing
+      // read hands lane j of the group the 4 consecutive k of row 16*(G%2) + j.
+      const int G = l >> 4, i = l & 15;
+#pragma unroll
+      for (int a = 0; a < NSUB; ++a) {
+        const int ch = (rowbase + a * 32) / 8 + 2 * (G & 1) + ((i & 3) >> 1);
+        off[a] = region + (8 * (G >> 1) + (i >> 2)) * 512 + ((ch ^ (((i >> 2) & 3) << 2)) << 4) + (i & 1) * 8;
+      }
+    }
+  }
+  __device__ __forceinline__ bf16x8 read(const unsigned char* smem, int a, int ks, int s) const {
+    if (!TR) {
+      return *reinterpret_cast<const bf16x8*>(smem + off[ks] + a * 32 * 64 + s * DL::TILE_BYTES);
+    } else {
+      typedef s16x4 __attribute__((address_space(3))) * lds_ptr_t;
+      const unsigned char* p = smem + off[a] + s * DL::TILE_BYTES + ks * 16 * 512;
+      s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(p));
+      s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(p + 4 * 512));
+      typedef short s16x8 __attribute__((ext_vector_type(8)));
+      s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      return __builtin_bit_cast(bf16x8, both);
+    }
+  }
+};
+
+template <typename TO, bool TA, bool TB, int EPI>
+__global__ __launch_bounds__(DL::NTHREADS, 2) void gemm_dl_kernel(const GemmParams p) {
+  using T = bf16_t;
+  constexpr int BM = DL::BM, BN = DL::BN, WM = DL::WM, WN = DL::WN, NSTAGE = DL::NSTAGE, TILE = DL::TILE_BYTES;
+  constexpr int MT = WM / 32, NT = WN / 32, WGN = BN / WN;
+  constexpr bool DUAL = (EPI == MVIT_EPI_SWIGLU);
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int total = tiles * p.split_k;
+  const int per_xcd = (total + 7) / 8;
+  const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (work >= total) return;
+  const int slice = work / tiles, tile = work % tiles;
+  const int tm = tile / p.tiles_n, tn = tile % p.tiles_n;
+  const int64_t k_begin = (int64_t)slice * p.k_chunk;
+  const int64_t k_end = p.split_k > 1 ? (k_begin + p.k_chunk < p.K ? k_begin + p.k_chunk : p.K) : p.K;
+  constexpr int N_PER_BLOCK = DUAL ? BN / 2 : BN;
+  const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * N_PER_BLOCK;
+
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wv / WGN, wn = wv % WGN;
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int a = 0; a < MT; ++a)
+#pragma unroll
+    for (int b = 0; b < NT; ++b)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
+
+  DlOperand<TA, false> la;
+  DlOperand<TB, DUAL> lb;
+  la.init(static_cast<const T*>(p.A), nullptr, p.lda, m0, p.M, k_begin, wv);
+  lb.init(static_cast<const T*>(p.B), static_cast<const T*>(p.B2), p.ldb, n0, p.N, k_begin, wv);
+  DlFrag<TA, MT> ra;
+  DlFrag<TB, NT> rb;
+  ra.init(wm * WM, 0);
+  rb.init(wn * WN, NSTAGE * TILE);
+
+  const int klen = (int)(k_end - k_begin);
+  const int T_ = (klen + DL::BK - 1) / DL::BK, k_tail = klen % DL::BK;
+  typedef __attribute__((address_space(3))) unsigned char lds_byte;
+  const unsigned lds0 = (unsigned)(__UINTPTR_TYPE__)(lds_byte*)smem_raw + wv * 2048;
+
+  auto issue = [&](int t, int s) {  // K tile t into stage s (both wave-uniform)
+    if (t >= T_) return;
+    if (k_tail != 0 && t == T_ - 1) {
+      la.issue_tail(smem_raw + s * TILE + wv * 2048, k_tail, wv);
+      lb.issue_tail(smem_raw + (NSTAGE + s) * TILE + wv * 2048, k_tail, wv);
+    } else {
+      la.issue(lds0 + s * TILE);
+      lb.issue(lds0 + (NSTAGE + s) * TILE);
+    }
+  };
+#pragma unroll
+  for (int t = 0; t < NSTAGE - 1; ++t) issue(t, t);
+
+  for (int t0 = 0; t0 < T_; t0 += NSTAGE) {
+#pragma unroll
+    for (int s = 0; s < NSTAGE; ++s) {
+      const int t = t0 + s;
+      if (t >= T_) break;
+      // tile t has landed once at most the loads of the min(rem, NSTAGE-2) younger tiles (4 per lane each) are pending
+      const int rem = T_ - 1 - t;
+      if (rem >= 2 && NSTAGE >= 4) wait_vm<8>();
+      else if (rem >= 1 && NSTAGE >= 3) wait_vm<4>();
+      else wait_vm<0>();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();  // every wave's share of tile t is in LDS; stage (s-1) has been consumed
+      issue(t + NSTAGE - 1, (s + NSTAGE - 1) % NSTAGE);
+
+      bf16x8 fa[2][MT], fb[2][NT];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+        for (int a = 0; a < MT; ++a) fa[ks][a] = ra.read(smem_raw, a, ks, s);
+#pragma unroll
+        for (int b = 0; b < NT; ++b) fb[ks][b] = rb.read(smem_raw, b, ks, s);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+          for (int b = 0; b < NT; ++b)
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks][a], fb[ks][b], acc[a][b], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+  __syncthreads();  // operands fully consumed before LDS is reused by the epilogue
+  run_epilogue<T, TO, EPI, BM, BN, WM, WN, DL::NTHREADS>(p, acc, smem_raw, m0, n0, wm, wn, slice);
+}
+
 // C[m, n] = sum over slices of the fp32 partial tiles (fixed order, so the result is reproducible).
 template <typename TO>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, int split_k, int64_t M, int64_t N,
@@ -491,9 +772,10 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 template <typename T, typename TO, bool TA, bool TB, int EPI, int VAR>
 int launch(const GemmParams& p, hipStream_t stream) {
   using W = Waves<VAR>;
-  using LA = TileLoader<T, BM, TA, W::NTHREADS, W::WN>;
-  using LB = TileLoader<T, BN, TB, W::NTHREADS, W::WN>;
-  const size_t operands = 2 * (size_t)(LA::LDS_ELEMS + LB::LDS_ELEMS) * sizeof(T);
+  constexpr int BM = W::BM, BN = W::BN;
+  using LA = TileLoader<T, BM, TA, W::NTHREADS, W::WN, false>;
+  using LB = TileLoader<T, BN, TB, W::NTHREADS, W::WN, false>;
+  const size_t operands = W::STAGES * (size_t)(LA::LDS_ELEMS + LB::LDS_ELEMS) * sizeof(T);
   const size_t staging = (size_t)(BM / W::WM) * 32 * (BN + 8) * sizeof(float);
   const size_t lds = operands > staging ? operands : staging;
   auto kern = gemm_kernel<T, TO, TA, TB, EPI, VAR>;
@@ -517,9 +799,39 @@ int launch(const GemmParams& p, hipStream_t stream) {
   return MVIT_OK;
 }
 
+template <typename TO, bool TA, bool TB, int EPI>
+int launch_dl(const GemmParams& p, hipStream_t stream) {
+  const size_t operands = 2 * (size_t)DL::NSTAGE * DL::TILE_BYTES;
+  const size_t staging = (size_t)(DL::BM / DL::WM) * 32 * (DL::BN + 8) * sizeof(float);
+  const size_t lds = operands > staging ? operands : staging;
+  auto kern = gemm_dl_kernel<TO, TA, TB, EPI>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return mvit_set_error(MVIT_ERR_LAUNCH, "gemm: hipFuncSetAttribute(%zu B LDS): %s", lds, hipGetErrorString(e));
+    attr_set = true;
+  }
+  if (p.split_k > 1 && EPI != MVIT_EPI_NONE) return mvit_set_error(MVIT_ERR_UNSUPPORTED, "gemm: split_k needs EPI_NONE");
+  const int total = p.tiles_m * p.tiles_n * p.split_k;
+  const int grid = ((total + 7) / 8) * 8;
+  hipLaunchKernelGGL(kern, grid, DL::NTHREADS, lds, stream, p);
+  MVIT_CHECK_LAUNCH("gemm");
+  if (p.split_k > 1) {
+    const int64_t elems = p.M * p.N;
+    const int rgrid = (int)((elems + 255) / 256 < 8192 ? (elems + 255) / 256 : 8192);
+    hipLaunchKernelGGL((splitk_reduce_kernel<TO>), rgrid, 256, 0, stream, p.workspace, p.split_k, p.M, p.N, static_cast<TO*>(p.C), p.ldc);
+    MVIT_CHECK_LAUNCH("gemm split-k reduce");
+  }
+  return MVIT_OK;
+}
+
 template <typename T, typename TO, bool TA, bool TB, int EPI>
 int launch_var(int var, const GemmParams& p, hipStream_t s) {
-  if (var == 1) return launch<T, TO, TA, TB, EPI, 1>(p, s);
+  if constexpr (sizeof(T) == 2) {
+    if (var == 3) return launch_dl<TO, TA, TB, EPI>(p, s);
+  }
+  if (var == 1 || var == 3) return launch<T, TO, TA, TB, EPI, 1>(p, s);
+  if (var == 2) return launch<T, TO, TA, TB, EPI, 2>(p, s);
   return launch<T, TO, TA, TB, EPI, 0>(p, s);
 }
 
@@ -594,6 +906,9 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
   const size_t es = a->dtype == MVIT_BF16 ? 2 : 4, eo = a->out_dtype == MVIT_BF16 ? 2 : 4;
   p.vec_ok = vec16(a->C, a->ldc, eo) && vec16(a->R, a->ldr, es) && vec16(a->aux, a->ldaux, es) && vec16(a->bias, 0, es) &&
              vec16(a->bias2, 0, es) && (a->aux_off * (int64_t)(es < eo ? es : eo)) % 16 == 0;
+  int var = (a->reserved >= 0 && a->reserved <= 3) ? a->reserved : 3;
+  if (var == 3 && (a->lda > (1ll << 22) || a->ldb > (1ll << 22))) var = 1;  // 32-bit lane offsets  // tile / wave layout, see Waves<>
+  const int BM = 256, BN = var == 2 ? 128 : 256;
   const int n_per_block = (epi == MVIT_EPI_SWIGLU) ? BN / 2 : BN;
   const int64_t tm = (a->M + BM - 1) / BM, tn = (a->N + n_per_block - 1) / n_per_block;
   MVIT_REQUIRE(tm * tn < (1ll << 30), "gemm: too many tiles");
@@ -609,7 +924,6 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
     MVIT_REQUIRE(tm * tn * slices < (1ll << 30), "gemm: too many tiles");
     if (slices > 1) { p.split_k = (int)slices; p.k_chunk = chunk; p.workspace = static_cast<float*>(a->workspace); }
   }
-  const int var = a->reserved == 1 ? 1 : 0;  // wave layout: 0 = 4 waves of 128x128, 1 = 8 waves of 128x64
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (a->dtype == MVIT_BF16) {
     if (a->out_dtype == MVIT_BF16) return dispatch_trans<bf16_t, bf16_t>(a->trans_a, a->trans_b, epi, var, p, s);
