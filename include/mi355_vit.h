@@ -134,7 +134,7 @@ typedef struct mvit_gemm_args {
   int trans_a;   /* 0: A is [M,K] (lda >= K);  1: A is [K,M] (lda >= M) */
   int trans_b;   /* 0: B is [N,K] (ldb >= K);  1: B is [K,N] (ldb >= N) */
   int epilogue;  /* MVIT_EPI_* */
-  int reserved;
+  int reserved;  /* main-loop variant: 0 = default (best known); 1..3 pick one explicitly (tuning / tests) */
   int64_t M, N, K;
   const void* A;
   int64_t lda;

@@ -1,15 +1,15 @@
 // MFMA GEMM for gfx950 with fused epilogues:  C[M,N] = epi( sum_k A[m,k] * B[n,k] ).
 //
-// Block tile 256x256.  Two wave layouts are built (selected by the host per problem):
-//   V0: 4 waves (2x2), each owning 128x128 as 4x4 MFMA 32x32 tiles (least LDS traffic per FLOP);
-//   V1: 8 waves (2x4), each owning 128x64  as 4x2 tiles (two waves per SIMD hide each other's LDS latency).
-//   bf16: v_mfma_f32_32x32x16_bf16, BK = 64.  Operands whose contraction index is contiguous in memory are
-//         staged as [row][k] and read with 16-byte LDS loads; operands whose contraction index is the slow
-//         dimension (dgrad's weight, both operands of wgrad) are staged as [k][row] exactly as they lie in
-//         memory and read with ds_read_b64_tr_b16, which hands each lane 4 consecutive k for its row.
-//   fp32: v_mfma_f32_32x32x2_f32, BK = 16 (parity mode; one LDS word per lane per MFMA operand).
-// LDS is double buffered: the next K tile travels global -> registers while the current one is consumed,
-// is written to the other buffer after the MFMAs, and one barrier per K step separates the two.
+// Main loops (selected by the host; mvit_gemm_args.reserved, 0 = default):
+//   3: bf16 default.  256x256 tile, 8 waves of 128x64 (4x2 MFMA 32x32x16 tiles each), BK = 32, four LDS stages
+//      filled by direct global -> LDS loads (see gemm_dl_kernel).
+//   1: 256x256 tile, 8 waves, BK = 64 (fp32: 16), global -> registers -> LDS, double-buffered LDS, one barrier
+//      per K step.  The fp32 parity path (v_mfma_f32_32x32x2_f32) and the fallback for huge leading dimensions.
+//   2: 256x128 tile, 4 waves, single LDS buffer, two work-groups per CU.
+// Operands whose contraction index is contiguous in memory are staged as [row][k] and read with 16-byte LDS
+// loads; operands whose contraction index is the slow dimension (dgrad's weight, both operands of wgrad) are
+// staged as [k][row] exactly as they lie in memory and read with ds_read_b64_tr_b16, which hands each lane 4
+// consecutive k for its row.
 // The epilogue stages the accumulators through LDS (fp32) so that bias / residual / activation inputs are
 // read and results written as 16-byte vectors along N.
 // Work-group ids are remapped so that the tiles a single XCD (one L2) works on are neighbours in N.
@@ -58,10 +58,6 @@ struct Cfg<float> {
 
 template <int VAR>
 struct Waves;
-template <>
-struct Waves<0> {  // 256x256 tile, 4 waves of 128x128, double-buffered LDS, one work-group per CU
-  static constexpr int BM = 256, BN = 256, WM = 128, WN = 128, NTHREADS = 256, STAGES = 2, MIN_WAVES = 1;
-};
 template <>
 struct Waves<1> {  // 256x256 tile, 8 waves of 128x64, double-buffered LDS, one work-group per CU
   static constexpr int BM = 256, BN = 256, WM = 128, WN = 64, NTHREADS = 512, STAGES = 2, MIN_WAVES = 2;
@@ -832,7 +828,7 @@ int launch_var(int var, const GemmParams& p, hipStream_t s) {
   }
   if (var == 1 || var == 3) return launch<T, TO, TA, TB, EPI, 1>(p, s);
   if (var == 2) return launch<T, TO, TA, TB, EPI, 2>(p, s);
-  return launch<T, TO, TA, TB, EPI, 0>(p, s);
+  return launch<T, TO, TA, TB, EPI, 1>(p, s);
 }
 
 template <typename T, typename TO, bool TA, bool TB>
@@ -906,7 +902,7 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
   const size_t es = a->dtype == MVIT_BF16 ? 2 : 4, eo = a->out_dtype == MVIT_BF16 ? 2 : 4;
   p.vec_ok = vec16(a->C, a->ldc, eo) && vec16(a->R, a->ldr, es) && vec16(a->aux, a->ldaux, es) && vec16(a->bias, 0, es) &&
              vec16(a->bias2, 0, es) && (a->aux_off * (int64_t)(es < eo ? es : eo)) % 16 == 0;
-  int var = (a->reserved >= 0 && a->reserved <= 3) ? a->reserved : 3;
+  int var = (a->reserved >= 1 && a->reserved <= 3) ? a->reserved : 3;  // 0 = default
   if (var == 3 && (a->lda > (1ll << 22) || a->ldb > (1ll << 22))) var = 1;  // 32-bit lane offsets  // tile / wave layout, see Waves<>
   const int BM = 256, BN = var == 2 ? 128 : 256;
   const int n_per_block = (epi == MVIT_EPI_SWIGLU) ? BN / 2 : BN;

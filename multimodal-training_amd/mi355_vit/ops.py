@@ -17,7 +17,7 @@ N_PARTIAL = 1024  # work-groups (= partial rows) of the RMSNorm backward: 4 per 
 
 import os as _os
 
-GEMM_VARIANT = int(_os.environ.get("MI355_VIT_GEMM_VARIANT", "3"))  # GEMM main loop (0: 4 waves, 1: 8 waves, 2: 256x128 tiles, 3: direct-to-LDS pipeline)
+GEMM_VARIANT = int(_os.environ.get("MI355_VIT_GEMM_VARIANT", "0"))  # GEMM main loop: 0 default, 1 register-staged, 2 256x128 tiles, 3 direct-to-LDS
 
 _trace = None  # optional list collecting (tag, info, start_event, end_event) per tagged launch
 
