@@ -152,8 +152,9 @@ typedef struct mvit_gemm_args {
   int64_t aux_off; /* column offset of the second half in aux (SWIGLU) / R and C (SWIGLU_BWD) */
   void* workspace; /* fp32 scratch of split_k * M * N floats when split_k > 1, else unused */
   int64_t workspace_bytes;
-  int split_k; /* <= 1: one work-group per tile walks all of K.  > 1 (EPI_NONE only): K is cut in split_k slices */
-  int reserved2; /*        whose fp32 partial tiles go to `workspace` and are summed by a second kernel (fixed order) */
+  int split_k;   /* <= 1: one work-group per tile walks all of K.  > 1 (EPI_NONE only): K is cut in split_k slices
+                    whose fp32 partial tiles go to `workspace` and are summed by a second kernel (fixed order) */
+  int reserved2; /* tile-order panel width: 0 = default; > 0 overrides (tuning) */
 } mvit_gemm_args;
 
 /* C[M,N] = epilogue(sum_k A[m,k] * B[n,k]).  Operands must be 16-byte aligned with lda/ldb multiples of

@@ -39,7 +39,25 @@ struct GemmParams {
   int64_t k_chunk;    // K extent of one slice (multiple of BK)
   float* workspace;   // [split_k][M][N] fp32 partial sums when split_k > 1
   int vec_ok;         // every epilogue pointer / stride allows 16-byte accesses
+  int panel_w;        // tiles are walked in panels of this many tile columns (M fastest across a panel's rows)
 };
+
+// Tile order inside one K slice: panels of panel_w tile columns; within a panel row by row.  Work-groups that run
+// at the same time on one XCD (consecutive tile indices) then cover a compact block of the output, e.g. 8 x 4
+// tiles, so the A and B panels they stream through that XCD's L2 are shared as widely as possible.
+__device__ __forceinline__ void tile_coords(const GemmParams& p, int tile, int& tm, int& tn) {
+  const int pw = p.panel_w;
+  const int full_panels = p.tiles_n / pw, per_panel = p.tiles_m * pw;
+  if (tile < full_panels * per_panel) {
+    const int r = tile % per_panel;
+    tm = r / pw;
+    tn = (tile / per_panel) * pw + r % pw;
+  } else {
+    const int r = tile - full_panels * per_panel, w = p.tiles_n - full_panels * pw;
+    tm = r / w;
+    tn = full_panels * pw + r % w;
+  }
+}
 
 template <typename T>
 struct Cfg;
@@ -434,7 +452,8 @@ __global__ __launch_bounds__(Waves<VAR>::NTHREADS, Waves<VAR>::MIN_WAVES) void g
   const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (work >= total) return;
   const int slice = work / tiles, tile = work % tiles;
-  const int tm = tile / p.tiles_n, tn = tile % p.tiles_n;
+  int tm, tn;
+  tile_coords(p, tile, tm, tn);
   const int64_t k_begin = (int64_t)slice * p.k_chunk;
   const int64_t k_end = p.split_k > 1 ? (k_begin + p.k_chunk < p.K ? k_begin + p.k_chunk : p.K) : p.K;
   constexpr int N_PER_BLOCK = DUAL ? BN / 2 : BN;
@@ -548,7 +567,7 @@ __global__ __launch_bounds__(Waves<VAR>::NTHREADS, Waves<VAR>::MIN_WAVES) void g
 // last K tile (K not a multiple of 32) is loaded through registers with zeros past the end of K.
 // The compiler does not see these loads: s_waitcnt vmcnt is placed by hand (loads return in order).
 struct DL {
-  static constexpr int BM = 256, BN = 256, BK = 32, WM = 128, WN = 64, NTHREADS = 512, NSTAGE = 4;
+  static constexpr int BM = 256, BN = 256, BK = 32, WM = 128, WN = 64, NTHREADS = 512;
   static constexpr int TILE_BYTES = 256 * BK * 2;
 };
 
@@ -618,6 +637,7 @@ struct DlOperand {
       if (k < k_rem) v = *reinterpret_cast<const bf16x8*>(base[i] + voff[i]);
       *reinterpret_cast<bf16x8*>(lds_slice + i * 1024 + l * 16) = v;
     }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // written before this wave's next barrier
   }
 };
 
@@ -657,10 +677,20 @@ struct DlFrag {
   }
 };
 
-template <typename TO, bool TA, bool TB, int EPI>
+// Wait until at most n K tiles' loads (4 per lane each) are still in flight.
+__device__ __forceinline__ void wait_tiles(int n) {
+  if (n >= 3) wait_vm<12>();
+  else if (n == 2) wait_vm<8>();
+  else if (n == 1) wait_vm<4>();
+  else wait_vm<0>();
+}
+
+// PF: the first 16-wide step's operands of tile t+1 are fetched from LDS while tile t's second step runs on the
+// MFMAs; tile t+1 must then have landed one barrier earlier, so one tile less is in flight.
+template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, bool PF>
 __global__ __launch_bounds__(DL::NTHREADS, 2) void gemm_dl_kernel(const GemmParams p) {
   using T = bf16_t;
-  constexpr int BM = DL::BM, BN = DL::BN, WM = DL::WM, WN = DL::WN, NSTAGE = DL::NSTAGE, TILE = DL::TILE_BYTES;
+  constexpr int BM = DL::BM, BN = DL::BN, WM = DL::WM, WN = DL::WN, TILE = DL::TILE_BYTES;
   constexpr int MT = WM / 32, NT = WN / 32, WGN = BN / WN;
   constexpr bool DUAL = (EPI == MVIT_EPI_SWIGLU);
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -671,7 +701,8 @@ __global__ __launch_bounds__(DL::NTHREADS, 2) void gemm_dl_kernel(const GemmPara
   const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (work >= total) return;
   const int slice = work / tiles, tile = work % tiles;
-  const int tm = tile / p.tiles_n, tn = tile % p.tiles_n;
+  int tm, tn;
+  tile_coords(p, tile, tm, tn);
   const int64_t k_begin = (int64_t)slice * p.k_chunk;
   const int64_t k_end = p.split_k > 1 ? (k_begin + p.k_chunk < p.K ? k_begin + p.k_chunk : p.K) : p.K;
   constexpr int N_PER_BLOCK = DUAL ? BN / 2 : BN;
@@ -715,38 +746,58 @@ __global__ __launch_bounds__(DL::NTHREADS, 2) void gemm_dl_kernel(const GemmPara
 #pragma unroll
   for (int t = 0; t < NSTAGE - 1; ++t) issue(t, t);
 
+  bf16x8 fa[2][MT], fb[2][NT];
+  if (PF && T_ > 0) {
+    wait_tiles(T_ - 1 < NSTAGE - 2 ? T_ - 1 : NSTAGE - 2);
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int a = 0; a < MT; ++a) fa[0][a] = ra.read(smem_raw, a, 0, 0);
+#pragma unroll
+    for (int b = 0; b < NT; ++b) fb[0][b] = rb.read(smem_raw, b, 0, 0);
+  }
   for (int t0 = 0; t0 < T_; t0 += NSTAGE) {
 #pragma unroll
     for (int s = 0; s < NSTAGE; ++s) {
       const int t = t0 + s;
       if (t >= T_) break;
-      // tile t has landed once at most the loads of the min(rem, NSTAGE-2) younger tiles (4 per lane each) are pending
-      const int rem = T_ - 1 - t;
-      if (rem >= 2 && NSTAGE >= 4) wait_vm<8>();
-      else if (rem >= 1 && NSTAGE >= 3) wait_vm<4>();
-      else wait_vm<0>();
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      __builtin_amdgcn_s_barrier();  // every wave's share of tile t is in LDS; stage (s-1) has been consumed
+      // tile t (PF: t+1) has landed once only the tiles issued after it are pending
+      const int rem = T_ - 1 - t - (PF ? 1 : 0);
+      constexpr int AHEAD = NSTAGE - 2 - (PF ? 1 : 0);
+      wait_tiles(rem < 0 ? 0 : (rem < AHEAD ? rem : AHEAD));
+      __builtin_amdgcn_s_barrier();  // every wave's share of that tile is in LDS; stage (s-1) has been consumed
       issue(t + NSTAGE - 1, (s + NSTAGE - 1) % NSTAGE);
 
-      bf16x8 fa[2][MT], fb[2][NT];
+      if (!PF) {
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
+        for (int a = 0; a < MT; ++a) fa[0][a] = ra.read(smem_raw, a, 0, s);
 #pragma unroll
-        for (int a = 0; a < MT; ++a) fa[ks][a] = ra.read(smem_raw, a, ks, s);
-#pragma unroll
-        for (int b = 0; b < NT; ++b) fb[ks][b] = rb.read(smem_raw, b, ks, s);
+        for (int b = 0; b < NT; ++b) fb[0][b] = rb.read(smem_raw, b, 0, s);
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
+      for (int a = 0; a < MT; ++a) fa[1][a] = ra.read(smem_raw, a, 1, s);
 #pragma unroll
-        for (int a = 0; a < MT; ++a)
+      for (int b = 0; b < NT; ++b) fb[1][b] = rb.read(smem_raw, b, 1, s);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int b = 0; b < NT; ++b)
-            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks][a], fb[ks][b], acc[a][b], 0, 0, 0);
+      for (int a = 0; a < MT; ++a)
+#pragma unroll
+        for (int b = 0; b < NT; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0][a], fb[0][b], acc[a][b], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (PF && t + 1 < T_) {
+#pragma unroll
+        for (int a = 0; a < MT; ++a) fa[0][a] = ra.read(smem_raw, a, 0, (s + 1) % NSTAGE);
+#pragma unroll
+        for (int b = 0; b < NT; ++b) fb[0][b] = rb.read(smem_raw, b, 0, (s + 1) % NSTAGE);
         __builtin_amdgcn_sched_barrier(0);
       }
+#pragma unroll
+      for (int a = 0; a < MT; ++a)
+#pragma unroll
+        for (int b = 0; b < NT; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][a], fb[1][b], acc[a][b], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
   __syncthreads();  // operands fully consumed before LDS is reused by the epilogue
@@ -795,12 +846,12 @@ int launch(const GemmParams& p, hipStream_t stream) {
   return MVIT_OK;
 }
 
-template <typename TO, bool TA, bool TB, int EPI>
+template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, bool PF>
 int launch_dl(const GemmParams& p, hipStream_t stream) {
-  const size_t operands = 2 * (size_t)DL::NSTAGE * DL::TILE_BYTES;
+  const size_t operands = 2 * (size_t)NSTAGE * DL::TILE_BYTES;
   const size_t staging = (size_t)(DL::BM / DL::WM) * 32 * (DL::BN + 8) * sizeof(float);
   const size_t lds = operands > staging ? operands : staging;
-  auto kern = gemm_dl_kernel<TO, TA, TB, EPI>;
+  auto kern = gemm_dl_kernel<TO, TA, TB, EPI, NSTAGE, PF>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -824,9 +875,10 @@ int launch_dl(const GemmParams& p, hipStream_t stream) {
 template <typename T, typename TO, bool TA, bool TB, int EPI>
 int launch_var(int var, const GemmParams& p, hipStream_t s) {
   if constexpr (sizeof(T) == 2) {
-    if (var == 3) return launch_dl<TO, TA, TB, EPI>(p, s);
+    if (var == 3) return launch_dl<TO, TA, TB, EPI, 4, false>(p, s);
+
   }
-  if (var == 1 || var == 3) return launch<T, TO, TA, TB, EPI, 1>(p, s);
+  if (var == 1 || var >= 3) return launch<T, TO, TA, TB, EPI, 1>(p, s);
   if (var == 2) return launch<T, TO, TA, TB, EPI, 2>(p, s);
   return launch<T, TO, TA, TB, EPI, 1>(p, s);
 }
@@ -903,12 +955,14 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
   p.vec_ok = vec16(a->C, a->ldc, eo) && vec16(a->R, a->ldr, es) && vec16(a->aux, a->ldaux, es) && vec16(a->bias, 0, es) &&
              vec16(a->bias2, 0, es) && (a->aux_off * (int64_t)(es < eo ? es : eo)) % 16 == 0;
   int var = (a->reserved >= 1 && a->reserved <= 3) ? a->reserved : 3;  // 0 = default
-  if (var == 3 && (a->lda > (1ll << 22) || a->ldb > (1ll << 22))) var = 1;  // 32-bit lane offsets  // tile / wave layout, see Waves<>
+  if (var >= 3 && (a->lda > (1ll << 22) || a->ldb > (1ll << 22))) var = 1;  // 32-bit lane offsets  // tile / wave layout, see Waves<>
   const int BM = 256, BN = var == 2 ? 128 : 256;
   const int n_per_block = (epi == MVIT_EPI_SWIGLU) ? BN / 2 : BN;
   const int64_t tm = (a->M + BM - 1) / BM, tn = (a->N + n_per_block - 1) / n_per_block;
   MVIT_REQUIRE(tm * tn < (1ll << 30), "gemm: too many tiles");
   p.tiles_m = (int)tm; p.tiles_n = (int)tn;
+  p.panel_w = tn <= 6 ? (int)tn : 4;
+  if (a->reserved2 > 0) p.panel_w = a->reserved2 < tn ? a->reserved2 : (int)tn;  // tuning override
   p.split_k = 1; p.k_chunk = a->K; p.workspace = nullptr;
   if (a->split_k > 1) {
     const int bk = a->dtype == MVIT_BF16 ? 64 : 16;

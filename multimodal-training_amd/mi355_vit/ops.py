@@ -17,6 +17,7 @@ N_PARTIAL = 1024  # work-groups (= partial rows) of the RMSNorm backward: 4 per 
 
 import os as _os
 
+GEMM_PANEL = int(_os.environ.get("MI355_VIT_GEMM_PANEL", "0"))  # tile-order panel width override (0: library default)
 GEMM_VARIANT = int(_os.environ.get("MI355_VIT_GEMM_VARIANT", "0"))  # GEMM main loop: 0 default, 1 register-staged, 2 256x128 tiles, 3 direct-to-LDS
 
 _trace = None  # optional list collecting (tag, info, start_event, end_event) per tagged launch
@@ -281,6 +282,7 @@ def gemm(
     args.dtype, args.out_dtype = dt(a), dt(out)
     args.trans_a, args.trans_b, args.epilogue, args.reserved = int(trans_a), int(trans_b), epilogue, GEMM_VARIANT
     args.M, args.N, args.K = M, N, K
+    args.reserved2 = GEMM_PANEL
     args.A, args.lda = a.data_ptr(), a.stride(0)
     args.B, args.ldb = b.data_ptr(), b.stride(0)
     if b2 is not None:
