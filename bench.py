@@ -74,7 +74,8 @@ def summarise_trace(records, cfg_kw, dtype):
         ent["launches"] += 1
         ent["ms"] += ms
         if tag.startswith("gemm"):
-            ent["flops"] += 2.0 * info["M"] * unpad.get(info["N"], info["N"]) * unpad.get(info["K"], info["K"])
+            halves = 2.0 if tag.endswith("epi4") else 1.0  # SWIGLU: N counts one of the two weight matrices
+            ent["flops"] += halves * 2.0 * info["M"] * unpad.get(info["N"], info["N"]) * unpad.get(info["K"], info["K"])
         elif tag.startswith("attn_fwd"):
             ent["flops"] += 4.0 * seg_sq_sum(info["cu"].cpu()) * info["head_dim"] * info["nheads"]
         elif tag.startswith("attn_bwd"):
@@ -91,19 +92,19 @@ def summarise_trace(records, cfg_kw, dtype):
 
 
 KERNEL_NAMES = {
-    "gemm_nn_epi0": "gemm_kernel<bf16, TO, TA=false, TB=false, EPI=NONE>",
-    "gemm_nn_epi1": "gemm_kernel<.., TA=false, TB=false, EPI=BIAS>",
-    "gemm_nn_epi2": "gemm_kernel<.., TA=false, TB=false, EPI=BIAS_RES>",
-    "gemm_nn_epi3": "gemm_kernel<.., TA=false, TB=false, EPI=BIAS_GELU>",
-    "gemm_nn_epi4": "gemm_kernel<.., TA=false, TB=false, EPI=SWIGLU>",
-    "gemm_nt_epi0": "gemm_kernel<.., TA=false, TB=true, EPI=NONE>",
-    "gemm_nt_epi5": "gemm_kernel<.., TA=false, TB=true, EPI=SWIGLU_BWD>",
-    "gemm_nt_epi6": "gemm_kernel<.., TA=false, TB=true, EPI=GELU_BWD>",
-    "gemm_tt_epi0": "gemm_kernel<.., TA=true, TB=true, EPI=NONE>",
+    "gemm_nn_epi0": "gemm_dl_kernel<TO, TA=false, TB=false, EPI=NONE>",
+    "gemm_nn_epi1": "gemm_dl_kernel<TO, TA=false, TB=false, EPI=BIAS>",
+    "gemm_nn_epi2": "gemm_dl_kernel<TO, TA=false, TB=false, EPI=BIAS_RES>",
+    "gemm_nn_epi3": "gemm_dl_kernel<TO, TA=false, TB=false, EPI=BIAS_GELU>",
+    "gemm_nn_epi4": "gemm_dl_kernel<TO, TA=false, TB=false, EPI=SWIGLU>",
+    "gemm_nt_epi0": "gemm_dl_kernel<TO, TA=false, TB=true, EPI=NONE>",
+    "gemm_nt_epi5": "gemm_dl_kernel<TO, TA=false, TB=true, EPI=SWIGLU_BWD>",
+    "gemm_nt_epi6": "gemm_dl_kernel<TO, TA=false, TB=true, EPI=GELU_BWD>",
+    "gemm_tt_epi0": "gemm_dl_kernel<TO, TA=true, TB=true, EPI=NONE>",
     "attn_fwd_full": "attn_fwd_mfma<5, 4, 32, true>",
-    "attn_bwd_full": "attn_delta_kernel + attn_bwd_dkdv_mfma<5, 4> + attn_bwd_dq_mfma<5, 4>",
+    "attn_bwd_full": "attn_delta_kernel + attn_bwd_dkdv_mfma<5, 8, 2> + attn_bwd_dq_mfma<5, 8, 2>",
     "attn_fwd_window": "attn_fwd_mfma<5, 1, 64, false>",
-    "attn_bwd_window": "attn_delta_kernel + attn_bwd_dkdv_mfma<5, 1> + attn_bwd_dq_mfma<5, 1>",
+    "attn_bwd_window": "attn_delta_kernel + attn_bwd_dkdv_mfma<5, 1, 4> + attn_bwd_dq_mfma<5, 1, 4>",
 }
 
 

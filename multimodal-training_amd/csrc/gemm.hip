@@ -566,10 +566,13 @@ __global__ __launch_bounds__(Waves<VAR>::NTHREADS, Waves<VAR>::MIN_WAVES) void g
 // Rows past the matrix edge are clamped to valid rows (they only feed outputs that are never stored).  A partial
 // last K tile (K not a multiple of 32) is loaded through registers with zeros past the end of K.
 // The compiler does not see these loads: s_waitcnt vmcnt is placed by hand (loads return in order).
+template <int NW>  // waves per work-group: 8 -> each owns 128x64 (two waves per SIMD), 4 -> 128x128 (one per SIMD)
 struct DL {
-  static constexpr int BM = 256, BN = 256, BK = 32, WM = 128, WN = 64, NTHREADS = 512;
+  static constexpr int BM = 256, BN = 256, BK = 32, WM = 128, WN = NW == 8 ? 64 : 128, NTHREADS = 64 * NW;
   static constexpr int TILE_BYTES = 256 * BK * 2;
+  static constexpr int CPT = 16 / NW;  // 1 KiB load instructions per wave, operand and K tile
 };
+constexpr int DL_BK = 32, DL_TILE_BYTES = 256 * DL_BK * 2;
 
 __device__ __forceinline__ void dl_load(unsigned lds_addr, unsigned voff, const char* base) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
@@ -579,51 +582,49 @@ __device__ __forceinline__ void wait_vm() {
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-template <bool TR, bool DUAL>
+template <bool TR, bool DUAL, int NW>
 struct DlOperand {
-  unsigned voff[2];     // byte offset of this lane's two 16-byte chunks from base[i]
-  const char* base[2];  // wave-uniform, advanced by `step` every K tile (DUAL: the two matrices)
+  static constexpr int CPT = DL<NW>::CPT, WN = DL<NW>::WN;
+  unsigned voff[CPT];  // byte offset of this lane's 16-byte chunks from `base`
+  const char* base;    // wave-uniform, advanced by `step` every K tile (DUAL: odd waves read the second matrix)
   int64_t step;
 
   __device__ __forceinline__ void init(const bf16_t* X, const bf16_t* X2, int64_t ld, int64_t row0, int64_t limit,
                                        int64_t k_begin, int wv) {
     const int l = threadIdx.x & 63;
-    step = TR ? 2 * DL::BK * ld : 2 * DL::BK;
+    step = TR ? 2 * DL_BK * ld : 2 * DL_BK;
+    // DUAL: tile row r = wn*WN + half*(WN/2) + j -> matrix `half`, row row0 + wn*(WN/2) + j; a wave's rows
+    // [wv * 16 * CPT, +16 * CPT) all have half = wv & 1.
+    const bf16_t* src = (DUAL && (wv & 1)) ? X2 : X;
+    base = reinterpret_cast<const char*>(TR ? src + k_begin * ld + row0 : src + row0 * ld + k_begin);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int q = wv * 2 + i;  // which 1 KiB of the stage this instruction fills
+    for (int i = 0; i < CPT; ++i) {
+      const int q = wv * CPT + i;  // which 1 KiB of the stage this instruction fills
       if (!TR) {
         const int r = q * 16 + (l >> 2), c = (l & 3) ^ ((r >> 2) & 3);
         int64_t grow = row0 + r;
-        const bf16_t* src = X;
-        if (DUAL) {  // tile row r = wn*WN + half*(WN/2) + j  ->  matrix `half` (uniform per wave), row row0 + wn*(WN/2) + j
-          grow = row0 + (r / DL::WN) * (DL::WN / 2) + (r % (DL::WN / 2));
-          if (wv & 1) src = X2;
-        }
+        if (DUAL) grow = row0 + (r / WN) * (WN / 2) + (r % (WN / 2));
         if (grow >= limit) grow = limit - 1;
         voff[i] = (unsigned)(((grow - row0) * ld + c * 8) * 2);
-        base[i] = reinterpret_cast<const char*>(src + row0 * ld + k_begin);
       } else {
         const int kr = 2 * q + (l >> 5);
         int ch = (l & 31) ^ ((kr & 3) << 2);
         if (row0 + ch * 8 >= limit) ch = 0;
         voff[i] = (unsigned)((kr * ld + ch * 8) * 2);
-        base[i] = reinterpret_cast<const char*>(X + k_begin * ld + row0);
       }
     }
   }
-  // lds_addr: LDS byte address of this wave's 2 KiB slice of the operand's stage
+  // lds_addr: LDS byte address of this wave's CPT KiB slice of the operand's stage
   __device__ __forceinline__ void issue(unsigned lds_addr) {
-    dl_load(lds_addr, voff[0], base[0]);
-    dl_load(lds_addr + 1024, voff[1], base[1]);
-    base[0] += step;
-    base[1] += step;
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) dl_load(lds_addr + i * 1024, voff[i], base);
+    base += step;
   }
   __device__ __forceinline__ void issue_tail(unsigned char* lds_slice, int k_rem, int wv) {
     const int l = threadIdx.x & 63;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int q = wv * 2 + i;
+    for (int i = 0; i < CPT; ++i) {
+      const int q = wv * CPT + i;
       int k;  // first contraction index of the chunk
       if (!TR) {
         const int r = q * 16 + (l >> 2);
@@ -634,7 +635,7 @@ struct DlOperand {
       bf16x8 v;
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] = from_f32<bf16_t>(0.f);
-      if (k < k_rem) v = *reinterpret_cast<const bf16x8*>(base[i] + voff[i]);
+      if (k < k_rem) v = *reinterpret_cast<const bf16x8*>(base + voff[i]);
       *reinterpret_cast<bf16x8*>(lds_slice + i * 1024 + l * 16) = v;
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // written before this wave's next barrier
@@ -664,10 +665,10 @@ struct DlFrag {
   }
   __device__ __forceinline__ bf16x8 read(const unsigned char* smem, int a, int ks, int s) const {
     if (!TR) {
-      return *reinterpret_cast<const bf16x8*>(smem + off[ks] + a * 32 * 64 + s * DL::TILE_BYTES);
+      return *reinterpret_cast<const bf16x8*>(smem + off[ks] + a * 32 * 64 + s * DL_TILE_BYTES);
     } else {
       typedef s16x4 __attribute__((address_space(3))) * lds_ptr_t;
-      const unsigned char* p = smem + off[a] + s * DL::TILE_BYTES + ks * 16 * 512;
+      const unsigned char* p = smem + off[a] + s * DL_TILE_BYTES + ks * 16 * 512;
       s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(p));
       s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(p + 4 * 512));
       typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -677,20 +678,22 @@ struct DlFrag {
   }
 };
 
-// Wait until at most n K tiles' loads (4 per lane each) are still in flight.
+// Wait until at most n K tiles' loads (PER per lane each) are still in flight.
+template <int PER>
 __device__ __forceinline__ void wait_tiles(int n) {
-  if (n >= 3) wait_vm<12>();
-  else if (n == 2) wait_vm<8>();
-  else if (n == 1) wait_vm<4>();
+  if (n >= 3) wait_vm<3 * PER>();
+  else if (n == 2) wait_vm<2 * PER>();
+  else if (n == 1) wait_vm<PER>();
   else wait_vm<0>();
 }
 
 // PF: the first 16-wide step's operands of tile t+1 are fetched from LDS while tile t's second step runs on the
 // MFMAs; tile t+1 must then have landed one barrier earlier, so one tile less is in flight.
-template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, bool PF>
-__global__ __launch_bounds__(DL::NTHREADS, 2) void gemm_dl_kernel(const GemmParams p) {
+template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, bool PF, int NW>
+__global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmParams p) {
   using T = bf16_t;
-  constexpr int BM = DL::BM, BN = DL::BN, WM = DL::WM, WN = DL::WN, TILE = DL::TILE_BYTES;
+  using D = DL<NW>;
+  constexpr int BM = D::BM, BN = D::BN, WM = D::WM, WN = D::WN, TILE = D::TILE_BYTES, SLICE = D::CPT * 1024;
   constexpr int MT = WM / 32, NT = WN / 32, WGN = BN / WN;
   constexpr bool DUAL = (EPI == MVIT_EPI_SWIGLU);
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -719,8 +722,8 @@ __global__ __launch_bounds__(DL::NTHREADS, 2) void gemm_dl_kernel(const GemmPara
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
-  DlOperand<TA, false> la;
-  DlOperand<TB, DUAL> lb;
+  DlOperand<TA, false, NW> la;
+  DlOperand<TB, DUAL, NW> lb;
   la.init(static_cast<const T*>(p.A), nullptr, p.lda, m0, p.M, k_begin, wv);
   lb.init(static_cast<const T*>(p.B), static_cast<const T*>(p.B2), p.ldb, n0, p.N, k_begin, wv);
   DlFrag<TA, MT> ra;
@@ -729,15 +732,15 @@ __global__ __launch_bounds__(DL::NTHREADS, 2) void gemm_dl_kernel(const GemmPara
   rb.init(wn * WN, NSTAGE * TILE);
 
   const int klen = (int)(k_end - k_begin);
-  const int T_ = (klen + DL::BK - 1) / DL::BK, k_tail = klen % DL::BK;
+  const int T_ = (klen + DL_BK - 1) / DL_BK, k_tail = klen % DL_BK;
   typedef __attribute__((address_space(3))) unsigned char lds_byte;
-  const unsigned lds0 = (unsigned)(__UINTPTR_TYPE__)(lds_byte*)smem_raw + wv * 2048;
+  const unsigned lds0 = (unsigned)(__UINTPTR_TYPE__)(lds_byte*)smem_raw + wv * SLICE;
 
   auto issue = [&](int t, int s) {  // K tile t into stage s (both wave-uniform)
     if (t >= T_) return;
     if (k_tail != 0 && t == T_ - 1) {
-      la.issue_tail(smem_raw + s * TILE + wv * 2048, k_tail, wv);
-      lb.issue_tail(smem_raw + (NSTAGE + s) * TILE + wv * 2048, k_tail, wv);
+      la.issue_tail(smem_raw + s * TILE + wv * SLICE, k_tail, wv);
+      lb.issue_tail(smem_raw + (NSTAGE + s) * TILE + wv * SLICE, k_tail, wv);
     } else {
       la.issue(lds0 + s * TILE);
       lb.issue(lds0 + (NSTAGE + s) * TILE);
@@ -748,7 +751,7 @@ __global__ __launch_bounds__(DL::NTHREADS, 2) void gemm_dl_kernel(const GemmPara
 
   bf16x8 fa[2][MT], fb[2][NT];
   if (PF && T_ > 0) {
-    wait_tiles(T_ - 1 < NSTAGE - 2 ? T_ - 1 : NSTAGE - 2);
+    wait_tiles<2 * D::CPT>(T_ - 1 < NSTAGE - 2 ? T_ - 1 : NSTAGE - 2);
     __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int a = 0; a < MT; ++a) fa[0][a] = ra.read(smem_raw, a, 0, 0);
@@ -763,7 +766,7 @@ __global__ __launch_bounds__(DL::NTHREADS, 2) void gemm_dl_kernel(const GemmPara
       // tile t (PF: t+1) has landed once only the tiles issued after it are pending
       const int rem = T_ - 1 - t - (PF ? 1 : 0);
       constexpr int AHEAD = NSTAGE - 2 - (PF ? 1 : 0);
-      wait_tiles(rem < 0 ? 0 : (rem < AHEAD ? rem : AHEAD));
+      wait_tiles<2 * D::CPT>(rem < 0 ? 0 : (rem < AHEAD ? rem : AHEAD));
       __builtin_amdgcn_s_barrier();  // every wave's share of that tile is in LDS; stage (s-1) has been consumed
       issue(t + NSTAGE - 1, (s + NSTAGE - 1) % NSTAGE);
 
@@ -801,7 +804,7 @@ __global__ __launch_bounds__(DL::NTHREADS, 2) void gemm_dl_kernel(const GemmPara
     }
   }
   __syncthreads();  // operands fully consumed before LDS is reused by the epilogue
-  run_epilogue<T, TO, EPI, BM, BN, WM, WN, DL::NTHREADS>(p, acc, smem_raw, m0, n0, wm, wn, slice);
+  run_epilogue<T, TO, EPI, BM, BN, WM, WN, D::NTHREADS>(p, acc, smem_raw, m0, n0, wm, wn, slice);
 }
 
 // C[m, n] = sum over slices of the fp32 partial tiles (fixed order, so the result is reproducible).
@@ -846,12 +849,13 @@ int launch(const GemmParams& p, hipStream_t stream) {
   return MVIT_OK;
 }
 
-template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, bool PF>
+template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, bool PF, int NW>
 int launch_dl(const GemmParams& p, hipStream_t stream) {
-  const size_t operands = 2 * (size_t)NSTAGE * DL::TILE_BYTES;
-  const size_t staging = (size_t)(DL::BM / DL::WM) * 32 * (DL::BN + 8) * sizeof(float);
+  using D = DL<NW>;
+  const size_t operands = 2 * (size_t)NSTAGE * D::TILE_BYTES;
+  const size_t staging = (size_t)(D::BM / D::WM) * 32 * (D::BN + 8) * sizeof(float);
   const size_t lds = operands > staging ? operands : staging;
-  auto kern = gemm_dl_kernel<TO, TA, TB, EPI, NSTAGE, PF>;
+  auto kern = gemm_dl_kernel<TO, TA, TB, EPI, NSTAGE, PF, NW>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -861,7 +865,7 @@ int launch_dl(const GemmParams& p, hipStream_t stream) {
   if (p.split_k > 1 && EPI != MVIT_EPI_NONE) return mvit_set_error(MVIT_ERR_UNSUPPORTED, "gemm: split_k needs EPI_NONE");
   const int total = p.tiles_m * p.tiles_n * p.split_k;
   const int grid = ((total + 7) / 8) * 8;
-  hipLaunchKernelGGL(kern, grid, DL::NTHREADS, lds, stream, p);
+  hipLaunchKernelGGL(kern, grid, D::NTHREADS, lds, stream, p);
   MVIT_CHECK_LAUNCH("gemm");
   if (p.split_k > 1) {
     const int64_t elems = p.M * p.N;
@@ -875,7 +879,7 @@ int launch_dl(const GemmParams& p, hipStream_t stream) {
 template <typename T, typename TO, bool TA, bool TB, int EPI>
 int launch_var(int var, const GemmParams& p, hipStream_t s) {
   if constexpr (sizeof(T) == 2) {
-    if (var == 3) return launch_dl<TO, TA, TB, EPI, 4, false>(p, s);
+    if (var == 3) return launch_dl<TO, TA, TB, EPI, 4, false, 8>(p, s);
 
   }
   if (var == 1 || var >= 3) return launch<T, TO, TA, TB, EPI, 1>(p, s);

@@ -4,6 +4,8 @@ all arithmetic happens in libmi355vit.so.  Every wrapper validates shapes on the
 from __future__ import annotations
 
 import ctypes as C
+import functools
+import os as _os
 from typing import Optional, Sequence, Tuple
 
 import torch
@@ -13,9 +15,6 @@ from ._lib import BF16, F32, GemmArgs
 
 _DT = {torch.float32: F32, torch.bfloat16: BF16}
 N_PARTIAL = 1024  # work-groups (= partial rows) of the RMSNorm backward: 4 per CU keep enough loads in flight
-
-
-import os as _os
 
 GEMM_PANEL = int(_os.environ.get("MI355_VIT_GEMM_PANEL", "0"))  # tile-order panel width override (0: library default)
 GEMM_VARIANT = int(_os.environ.get("MI355_VIT_GEMM_VARIANT", "0"))  # GEMM main loop: 0 default, 1 register-staged, 2 256x128 tiles, 3 direct-to-LDS
@@ -319,11 +318,32 @@ def gemm(
     return out
 
 
+_N_CU = 256  # MI355X compute units; one 256x256 GEMM work-group runs per CU
+
+
+@functools.lru_cache(maxsize=None)
 def wgrad_split_k(out_rows: int, out_cols: int, k: int) -> int:
-    """K slices for a weight-gradient GEMM: few output tiles (256x256) but a long contraction (the tokens)."""
+    """K slices for a weight-gradient GEMM: few output tiles (256x256) but a long contraction (the tokens).
+
+    Picks the slice count with the lowest modelled time.  Work items (tiles x slices) run in rounds of one per
+    CU, so the count should fill whole rounds; every slice costs an fp32 partial tile that a second kernel
+    re-reads.  Constants are microseconds measured on MI355X (a 32-deep K step takes 0.6 us on a lightly loaded
+    chip, 0.95 us when every CU is busy; ~8 us per tile epilogue; ~3.5 TB/s for the partial-sum traffic)."""
     tiles = -(-out_rows // 256) * -(-out_cols // 256)
-    want = max(1, min(16, round(768 / tiles)))
-    return max(1, min(want, k // 512))
+    best, best_t = 1, None
+    for sk in range(1, 17):
+        if sk > 1 and k // sk < 512:
+            break
+        items = tiles * sk
+        rounds = -(-items // _N_CU)
+        load = items / (rounds * _N_CU)
+        steps = -(-(-(-k // sk)) // 64) * 2
+        t = rounds * (steps * (0.6 + 0.35 * load) + 8.0)
+        if sk > 1:
+            t += 5.0 + sk * out_rows * out_cols * 4 / 3.5e6
+        if best_t is None or t < best_t:
+            best, best_t = sk, t
+    return best
 
 
 # ------------------------------------------------------------------------------ attention
