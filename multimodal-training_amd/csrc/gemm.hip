@@ -107,6 +107,11 @@ __device__ __forceinline__ void load8(const float* p, float* v) {
     v[4 + e] = b[e];
   }
 }
+template <typename T>
+__device__ __forceinline__ void unpack8(const T __attribute__((ext_vector_type(8))) & x, float* v) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = (float)x[e];
+}
 __device__ __forceinline__ void store8(bf16_t* p, const float* v) {
   bf16x8 x;
 #pragma unroll
@@ -245,8 +250,10 @@ __device__ __forceinline__ float frag_f32(const float* lds, int row, int k) {
 // Epilogue on 8 consecutive output columns n..n+7 of row m.  v: accumulators (gate half for SWIGLU), u: up half.
 // FULL: all 8 columns exist and every pointer allows 16-byte accesses (compile-time trip counts, vector memory
 // operations); otherwise a scalar path bounded by the matrix edge.
-template <typename T, typename TO, int EPI, bool FULL>
-__device__ __forceinline__ void emit8_impl(const GemmParams& p, int64_t m, int64_t n, float* v, const float* u) {
+// PRE: the epilogue's per-element inputs (residual / saved activations) were fetched earlier into pre[0..1].
+template <typename T, typename TO, int EPI, bool FULL, bool PRE = false>
+__device__ __forceinline__ void emit8_impl(const GemmParams& p, int64_t m, int64_t n, float* v, const float* u,
+                                           const T __attribute__((ext_vector_type(8))) * pre = nullptr) {
   TO* Cp = static_cast<TO*>(p.C);
   const T* Rp = static_cast<const T*>(p.R);
   T* auxp = static_cast<T*>(p.aux);
@@ -300,7 +307,10 @@ __device__ __forceinline__ void emit8_impl(const GemmParams& p, int64_t m, int64
     const T* g_in = Rp + m * p.ldr + n;
     const T* u_in = g_in + p.aux_off;
     float g[8], uu[8], dg[8], du[8];
-    if (vec) {
+    if (PRE) {
+      unpack8<T>(pre[0], g);
+      unpack8<T>(pre[1], uu);
+    } else if (vec) {
       load8(g_in, g);
       load8(u_in, uu);
     } else {
@@ -330,7 +340,8 @@ __device__ __forceinline__ void emit8_impl(const GemmParams& p, int64_t m, int64
   }
   if constexpr (EPI == MVIT_EPI_BIAS_RES || EPI == MVIT_EPI_GELU_BWD) {
     float r[8];
-    if (vec) load8(Rp + m * p.ldr + n, r);
+    if (PRE) unpack8<T>(pre[0], r);
+    else if (vec) load8(Rp + m * p.ldr + n, r);
     else
       for (int e = 0; e < 8; ++e) r[e] = e < cnt ? to_f32(Rp[m * p.ldr + n + e]) : 0.f;
     for (int e = 0; e < 8; ++e) {
@@ -383,6 +394,51 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
   const bool to_ws = (EPI == MVIT_EPI_NONE) && p.split_k > 1;
   float* ws = to_ws ? p.workspace + (int64_t)slice * p.M * p.N : nullptr;
   const bool ws_vec = (p.N % 4 == 0);
+
+  // Tiles inside the matrix whose epilogue reads one value per output element: those reads are issued one pass
+  // ahead, so their latency hides behind the LDS staging and the previous pass's arithmetic and stores.
+  constexpr bool HAS_IN = (EPI == MVIT_EPI_BIAS_RES || EPI == MVIT_EPI_GELU_BWD || EPI == MVIT_EPI_SWIGLU_BWD);
+  if constexpr (HAS_IN && (PASS_ROWS * GROUPS) % NTHREADS == 0) {
+    if (p.vec_ok && m0 + BM <= p.M && n0 + NCOLS <= p.N) {
+      constexpr int ITEMS = PASS_ROWS * GROUPS / NTHREADS, NLOAD = EPI == MVIT_EPI_SWIGLU_BWD ? 2 : 1;
+      typedef T raw8 __attribute__((ext_vector_type(8)));
+      const T* Rp = static_cast<const T*>(p.R);
+      raw8 pre[2][ITEMS][NLOAD];
+      auto fetch = [&](int a, raw8(&dst)[ITEMS][NLOAD]) {
+#pragma unroll
+        for (int it = 0; it < ITEMS; ++it) {
+          const int c = threadIdx.x + NTHREADS * it, row = c / GROUPS, cg = c % GROUPS;
+          const T* r = Rp + (m0 + (row / 32) * WM + a * 32 + (row % 32)) * p.ldr + n0 + cg * 8;
+          dst[it][0] = *reinterpret_cast<const raw8*>(r);
+          if (NLOAD == 2) dst[it][1] = *reinterpret_cast<const raw8*>(r + p.aux_off);
+        }
+      };
+      fetch(0, pre[0]);
+#pragma unroll
+      for (int a = 0; a < MT; ++a) {
+        if (a > 0) __syncthreads();
+#pragma unroll
+        for (int b = 0; b < NT; ++b) {
+          const int col = wn * WN + b * 32 + lc;
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) stage[(wm * 32 + 8 * j + lr + i) * SP + col] = acc[a][b][4 * j + i];
+        }
+        __syncthreads();
+        if (a + 1 < MT) fetch(a + 1, pre[(a + 1) & 1]);
+#pragma unroll
+        for (int it = 0; it < ITEMS; ++it) {
+          const int c = threadIdx.x + NTHREADS * it, row = c / GROUPS, cg = c % GROUPS;
+          const float* sp = stage + row * SP + cg * 8;
+          const f32x4 v0 = *reinterpret_cast<const f32x4*>(sp), v1 = *reinterpret_cast<const f32x4*>(sp + 4);
+          float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+          emit8_impl<T, TO, EPI, true, true>(p, m0 + (row / 32) * WM + a * 32 + (row % 32), n0 + cg * 8, v, nullptr, pre[a & 1][it]);
+        }
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int a = 0; a < MT; ++a) {
     if (a > 0) __syncthreads();
