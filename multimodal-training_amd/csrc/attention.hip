@@ -372,6 +372,39 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const T* __restrict__ o
   delta[(int64_t)h * total + s] = acc;
 }
 
+// Same result with coalesced traffic: a block takes 16 consecutive rows; every thread multiplies 16-byte chunks
+// (consecutive threads, consecutive chunks of a row), parks the chunk sums in LDS, and thread (h, r) then adds the
+// chunks of its head in a fixed order and writes delta[h][s0 + r], 16 consecutive floats per head.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_delta_rows_kernel(const T* __restrict__ o, const T* __restrict__ d_o,
+                                                              float* __restrict__ delta, int64_t total, int nheads, int hd,
+                                                              int64_t o_stride, int64_t do_stride) {
+  constexpr int V = mvit_elem<T>::vec, R = 16;
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  extern __shared__ float part[];  // [R][nheads * hd / V]
+  const int cph = hd / V, cpr = nheads * cph;
+  const int64_t s0 = (int64_t)blockIdx.x * R;
+  const int rows = total - s0 < R ? (int)(total - s0) : R;
+  for (int q = threadIdx.x; q < rows * cpr; q += 256) {
+    const int r = q / cpr, c = q % cpr;
+    const vec_t x = *reinterpret_cast<const vec_t*>(o + (s0 + r) * o_stride + (int64_t)c * V);
+    const vec_t y = *reinterpret_cast<const vec_t*>(d_o + (s0 + r) * do_stride + (int64_t)c * V);
+    float acc = 0.f;
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc += to_f32(x[e]) * to_f32(y[e]);
+    part[q] = acc;
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < nheads * R; t += 256) {
+    const int h = t / R, r = t % R;
+    if (r >= rows) continue;
+    const float* src = part + r * cpr + h * cph;
+    float acc = 0.f;
+    for (int j = 0; j < cph; ++j) acc += src[j];
+    delta[(int64_t)h * total + s0 + r] = acc;
+  }
+}
+
 // ================================================================================================
 // dK, dV.  Block = 64*NWAVES keys of one (segment, head); 32 queries per iteration, Q / dO tiles (and the
 // rows' lse, delta) double buffered in LDS with the next tile's loads in flight during the MFMAs.
@@ -929,12 +962,22 @@ int mvit_attn_bwd(const void* q, const void* k, const void* v, const void* o, co
   p.q_stride = q_stride; p.k_stride = k_stride; p.v_stride = v_stride; p.o_stride = o_stride; p.do_stride = do_stride;
   p.dq_stride = dq_stride; p.dk_stride = dk_stride; p.dv_stride = dv_stride; p.scale = scale;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  const int64_t npairs = total * nheads;
-  const int dgrid = (int)((npairs + 255) / 256);
-  if (dtype == MVIT_BF16)
-    hipLaunchKernelGGL((attn_delta_kernel<bf16_t>), dgrid, 256, 0, s, (const bf16_t*)o, (const bf16_t*)d_o, delta, total, nheads, head_dim, o_stride, do_stride);
-  else
-    hipLaunchKernelGGL((attn_delta_kernel<float>), dgrid, 256, 0, s, (const float*)o, (const float*)d_o, delta, total, nheads, head_dim, o_stride, do_stride);
+  const int vecw = dtype == MVIT_BF16 ? 8 : 4;
+  const size_t part_bytes = (size_t)16 * nheads * (head_dim / vecw) * sizeof(float);
+  if (head_dim % vecw == 0 && o_stride % vecw == 0 && do_stride % vecw == 0 && part_bytes <= 48 * 1024 && mvit_aligned16(o) && mvit_aligned16(d_o)) {
+    const int dgrid = (int)((total + 15) / 16);
+    if (dtype == MVIT_BF16)
+      hipLaunchKernelGGL((attn_delta_rows_kernel<bf16_t>), dgrid, 256, part_bytes, s, (const bf16_t*)o, (const bf16_t*)d_o, delta, total, nheads, head_dim, o_stride, do_stride);
+    else
+      hipLaunchKernelGGL((attn_delta_rows_kernel<float>), dgrid, 256, part_bytes, s, (const float*)o, (const float*)d_o, delta, total, nheads, head_dim, o_stride, do_stride);
+  } else {
+    const int64_t npairs = total * nheads;
+    const int dgrid = (int)((npairs + 255) / 256);
+    if (dtype == MVIT_BF16)
+      hipLaunchKernelGGL((attn_delta_kernel<bf16_t>), dgrid, 256, 0, s, (const bf16_t*)o, (const bf16_t*)d_o, delta, total, nheads, head_dim, o_stride, do_stride);
+    else
+      hipLaunchKernelGGL((attn_delta_kernel<float>), dgrid, 256, 0, s, (const float*)o, (const float*)d_o, delta, total, nheads, head_dim, o_stride, do_stride);
+  }
   MVIT_CHECK_LAUNCH("attn_delta");
   if (dtype == MVIT_BF16) {
     switch (head_dim) {

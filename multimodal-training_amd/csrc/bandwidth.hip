@@ -151,6 +151,30 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __res
   }
 }
 
+// The same sum for cols % 4 == 0: a block owns 16 columns (4 lanes x float4) and 64 row groups, so that a tall
+// partial array (1024 rows from the RMSNorm backward) is walked by many short, independent load chains.
+template <typename T>
+__global__ __launch_bounds__(256) void reduce_partials_vec_kernel(const float* __restrict__ partial, int n_partial,
+                                                                  int64_t cols, T* __restrict__ out) {
+  __shared__ float red[64][17];
+  const int cx = threadIdx.x & 3, ry = threadIdx.x >> 2;
+  const int64_t c = (int64_t)blockIdx.x * 16 + cx * 4;
+  f32x4 s = {0.f, 0.f, 0.f, 0.f};
+  if (c < cols) {
+#pragma unroll 4
+    for (int b = ry; b < n_partial; b += 64) s += *reinterpret_cast<const f32x4*>(partial + (size_t)b * cols + c);
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) red[ry][cx * 4 + e] = s[e];
+  __syncthreads();
+  if (threadIdx.x < 16 && (int64_t)blockIdx.x * 16 + threadIdx.x < cols) {
+    float t = 0.f;
+#pragma unroll
+    for (int k = 0; k < 64; ++k) t += red[k][threadIdx.x];
+    out[(int64_t)blockIdx.x * 16 + threadIdx.x] = from_f32<T>(t);
+  }
+}
+
 // Column sums with 16-byte loads: a block owns 128 columns (16 lanes x 8/4 elements) and 16 row phases.
 template <typename T>
 __global__ __launch_bounds__(256) void colsum_vec_kernel(const T* __restrict__ x, int64_t ld, int64_t rows, int64_t cols,
@@ -363,6 +387,15 @@ int mvit_rmsnorm_bwd(const void* dy, const void* x, const void* w, const float* 
 
 int mvit_reduce_partials(const float* partial, int n_partial, int64_t cols, void* out, int out_dtype, mvit_stream_t stream) {
   MVIT_REQUIRE(partial && out && n_partial > 0 && cols > 0, "reduce_partials: bad arguments");
+  if (cols % 4 == 0 && mvit_aligned16(partial) && (out_dtype == MVIT_BF16 || out_dtype == MVIT_F32)) {
+    const int vgrid = (int)((cols + 15) / 16);
+    if (out_dtype == MVIT_BF16)
+      hipLaunchKernelGGL((reduce_partials_vec_kernel<bf16_t>), vgrid, 256, 0, S_(stream), partial, n_partial, cols, (bf16_t*)out);
+    else
+      hipLaunchKernelGGL((reduce_partials_vec_kernel<float>), vgrid, 256, 0, S_(stream), partial, n_partial, cols, (float*)out);
+    MVIT_CHECK_LAUNCH("reduce_partials");
+    return MVIT_OK;
+  }
   const int grid = (int)((cols + 31) / 32);
   if (out_dtype == MVIT_BF16)
     hipLaunchKernelGGL((reduce_partials_kernel<bf16_t>), grid, 256, 0, S_(stream), partial, n_partial, cols, (bf16_t*)out);
