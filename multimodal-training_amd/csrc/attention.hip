@@ -676,6 +676,202 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams
 }
 
 // ================================================================================================
+// Whole backward of a short segment (<= 64 rows, the windowed layers) in one wave: Q, K, V and dO of one
+// (segment, head) are staged in LDS once.  Pass A works in the dQ orientation (a lane owns a query), where
+// delta_q = sum_k P[q,k] * dP[q,k] (equal to dO_q . O_q, so O is never read) is a lane-local sum, and writes dQ;
+// pass B repeats the dK/dV kernel's tile loop on the staged tiles.  HBM traffic: four tiles in, three out.
+template <int ND>
+__global__ __launch_bounds__(64) void attn_bwd_window_mfma(const AttnParams p) {
+  using G = Geo<ND>;
+  constexpr int HD = G::HD, R = 64, PK = G::PK;
+  __shared__ __attribute__((aligned(16))) bf16_t lds_q[R * PK];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_k[R * PK];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_v[R * PK];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_do[R * PK];
+  __shared__ __attribute__((aligned(16))) float lds_lse[R];
+  __shared__ __attribute__((aligned(16))) float lds_delta[R];
+
+  const int seg = blockIdx.y, h = blockIdx.z;
+  const int s0 = p.cu[seg];
+  const int L = min(p.cu[seg + 1] - s0, R);
+  if (L <= 0) return;
+  const int l = threadIdx.x, g = l >> 4, r = l & 15;
+  const float c = p.scale * LOG2E;
+  {
+    TileStager<ND, R, PK, 64> sq, sk, sv, sdo;
+    sq.init(p.q_stride);
+    sk.init(p.k_stride);
+    sv.init(p.v_stride);
+    sdo.init(p.do_stride);
+    sq.load(static_cast<const bf16_t*>(p.q) + (int64_t)s0 * p.q_stride + (int64_t)h * HD, L);
+    sk.load(static_cast<const bf16_t*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD, L);
+    sv.load(static_cast<const bf16_t*>(p.v) + (int64_t)s0 * p.v_stride + (int64_t)h * HD, L);
+    sdo.load(static_cast<const bf16_t*>(p.d_o) + (int64_t)s0 * p.do_stride + (int64_t)h * HD, L);
+    lds_lse[l] = l < L ? p.lse[(int64_t)h * p.total + s0 + l] * LOG2E : INFINITY;  // +inf => p = 0 for padded queries
+    sq.store(lds_q);
+    sk.store(lds_k);
+    sv.store(lds_v);
+    sdo.store(lds_do);
+  }
+  __syncthreads();
+
+  // ---- pass A: dQ^T += K^T dS^T per 16-query block, keys in two chunks of 32
+  {
+    RowFrag<ND> ka[2][2], va[2][2];
+    bf16x8 kt[2][ND];
+#pragma unroll
+    for (int kc = 0; kc < 2; ++kc) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        load_rowfrag_lds<ND, PK>(ka[kc][t], lds_k, kc * 32 + t * 16 + r, g);
+        load_rowfrag_lds<ND, PK>(va[kc][t], lds_v, kc * 32 + t * 16 + r, g);
+      }
+#pragma unroll
+      for (int d = 0; d < ND; ++d) {
+        const int off = (kc * 32 + 4 * g + (r >> 2)) * PK + 16 * d + 4 * (r & 3);
+        kt[kc][d] = tr_pair(lds_k + off, lds_k + off + 16 * PK);
+      }
+    }
+    bf16_t* DQ = static_cast<bf16_t*>(p.dq) + (int64_t)s0 * p.dq_stride + (int64_t)h * HD;
+    float* DELTA = p.delta + (int64_t)h * p.total + s0;
+#pragma unroll 1
+    for (int qb = 0; qb < 4; ++qb) {
+      if (qb * 16 >= L) break;
+      const int qi = qb * 16 + r;
+      RowFrag<ND> qf, dof;
+      load_rowfrag_lds<ND, PK>(qf, lds_q, qi, g);
+      load_rowfrag_lds<ND, PK>(dof, lds_do, qi, g);
+      const float neg_lse2 = -lds_lse[qi];
+      f32x4 e[2][2], dp[2][2];
+      float part = 0.f;
+#pragma unroll
+      for (int kc = 0; kc < 2; ++kc)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const f32x4 sc = dot_frag<ND>(ka[kc][t], qf);  // S[q = qb*16+r][key = kc*32+t*16+4g+i]
+          dp[kc][t] = dot_frag<ND>(va[kc][t], dof);      // dP, same layout
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float x = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], c, neg_lse2));
+            if (kc * 32 + t * 16 + 4 * g + i >= L) x = 0.f;  // keys past the segment end
+            e[kc][t][i] = x;
+            part = __builtin_fmaf(x, dp[kc][t][i], part);
+          }
+        }
+      part += __shfl_xor(part, 16);
+      part += __shfl_xor(part, 32);  // lanes r, r+16, r+32, r+48 share query qb*16+r
+      if (g == 0) {
+        lds_delta[qi] = part;
+        if (qi < L) DELTA[qi] = part;
+      }
+      f32x4 dq[ND];
+#pragma unroll
+      for (int d = 0; d < ND; ++d) dq[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kc = 0; kc < 2; ++kc) {
+        f32x4 ds[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) ds[t][i] = e[kc][t][i] * (dp[kc][t][i] - part);
+        const bf16x8 dsb = pack8(ds[0], ds[1]);
+#pragma unroll
+        for (int d = 0; d < ND; ++d) dq[d] = mfma32(kt[kc][d], dsb, dq[d]);
+      }
+      if (qi < L) {
+#pragma unroll
+        for (int d = 0; d < ND; ++d) {
+          bf16x4 a;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) a[i] = (bf16_t)(dq[d][i] * p.scale);
+          *reinterpret_cast<bf16x4*>(DQ + (int64_t)qi * p.dq_stride + 16 * d + 4 * g) = a;
+        }
+      }
+    }
+    for (int q = 16 * ((L + 15) / 16) + l; q < R; q += 64) lds_delta[q] = 0.f;  // query blocks that were skipped
+  }
+  __syncthreads();
+
+  // ---- pass B: dV^T += dO^T P, dK^T += Q^T dS per 16-key block, queries in two tiles of 32
+  {
+    RowFrag<ND> kf[4], vf[4];
+    f32x4 dk[4][ND], dv[4][ND];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      load_rowfrag_lds<ND, PK>(kf[kb], lds_k, kb * 16 + r, g);
+      load_rowfrag_lds<ND, PK>(vf[kb], lds_v, kb * 16 + r, g);
+#pragma unroll
+      for (int d = 0; d < ND; ++d) {
+        dk[kb][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dv[kb][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+#pragma unroll 1
+    for (int qs = 0; qs < L; qs += 32) {
+      const bf16_t* tq = lds_q + qs * PK;
+      const bf16_t* tdo = lds_do + qs * PK;
+      RowFrag<ND> qa[2], da[2];
+      bf16x8 qt[ND], dt_[ND];
+      f32x4 lse2[2], dl[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        load_rowfrag_lds<ND, PK>(qa[t], tq, t * 16 + r, g);
+        load_rowfrag_lds<ND, PK>(da[t], tdo, t * 16 + r, g);
+        lse2[t] = *reinterpret_cast<const f32x4*>(lds_lse + qs + t * 16 + 4 * g);
+        dl[t] = *reinterpret_cast<const f32x4*>(lds_delta + qs + t * 16 + 4 * g);
+      }
+#pragma unroll
+      for (int d = 0; d < ND; ++d) {
+        const int off = (4 * g + (r >> 2)) * PK + 16 * d + 4 * (r & 3);
+        qt[d] = tr_pair(tq + off, tq + off + 16 * PK);
+        dt_[d] = tr_pair(tdo + off, tdo + off + 16 * PK);
+      }
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        f32x4 pv[2], ds[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const f32x4 sc = dot_frag<ND>(qa[t], kf[kb]);   // S[q = qs+t*16+4g+i][key = kb*16+r]
+          const f32x4 dpp = dot_frag<ND>(da[t], vf[kb]);  // dP, same layout
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float x = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], c, -lse2[t][i]));
+            pv[t][i] = x;
+            ds[t][i] = x * (dpp[i] - dl[t][i]);
+          }
+        }
+        const bf16x8 pb = pack8(pv[0], pv[1]);
+        const bf16x8 dsb = pack8(ds[0], ds[1]);
+#pragma unroll
+        for (int d = 0; d < ND; ++d) {
+          dv[kb][d] = mfma32(dt_[d], pb, dv[kb][d]);
+          dk[kb][d] = mfma32(qt[d], dsb, dk[kb][d]);
+        }
+      }
+    }
+    bf16_t* DK = static_cast<bf16_t*>(p.dk) + (int64_t)s0 * p.dk_stride + (int64_t)h * HD;
+    bf16_t* DV = static_cast<bf16_t*>(p.dv) + (int64_t)s0 * p.dv_stride + (int64_t)h * HD;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      const int ki = kb * 16 + r;
+      if (ki < L) {
+#pragma unroll
+        for (int d = 0; d < ND; ++d) {
+          bf16x4 a, b;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            a[i] = (bf16_t)(dk[kb][d][i] * p.scale);
+            b[i] = (bf16_t)dv[kb][d][i];
+          }
+          *reinterpret_cast<bf16x4*>(DK + (int64_t)ki * p.dk_stride + 16 * d + 4 * g) = a;
+          *reinterpret_cast<bf16x4*>(DV + (int64_t)ki * p.dv_stride + 16 * d + 4 * g) = b;
+        }
+      }
+    }
+  }
+}
+
+// ================================================================================================
 // fp32 parity kernels: one lane per row, 32-row tiles of the other side broadcast from LDS.
 template <int HD>
 __global__ __launch_bounds__(64) void attn_fwd_f32(const AttnParams p) {
@@ -875,8 +1071,12 @@ int launch_bwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
   // short segments (windows): one wave owns a whole 64-row block; long ones: 8 waves x 32 rows (2 waves per SIMD)
   if (max_seqlen <= 64) {
     dim3 grid(1, (unsigned)n_seg, (unsigned)p.nheads);
-    hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 1, 4>), grid, 64, 0, s, p);
-    hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 1, 4>), grid, 64, 0, s, p);
+    if constexpr (ND <= 5) {
+      hipLaunchKernelGGL((attn_bwd_window_mfma<ND>), grid, 64, 0, s, p);  // computes delta itself
+    } else {
+      hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 1, 4>), grid, 64, 0, s, p);
+      hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 1, 4>), grid, 64, 0, s, p);
+    }
   } else if (max_seqlen <= 128) {
     dim3 grid(1, (unsigned)n_seg, (unsigned)p.nheads);
     hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 2, 4>), grid, 128, 0, s, p);
@@ -964,7 +1164,9 @@ int mvit_attn_bwd(const void* q, const void* k, const void* v, const void* o, co
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const int vecw = dtype == MVIT_BF16 ? 8 : 4;
   const size_t part_bytes = (size_t)16 * nheads * (head_dim / vecw) * sizeof(float);
-  if (head_dim % vecw == 0 && o_stride % vecw == 0 && do_stride % vecw == 0 && part_bytes <= 48 * 1024 && mvit_aligned16(o) && mvit_aligned16(d_o)) {
+  if (dtype == MVIT_BF16 && max_seqlen <= 64 && head_dim <= 80) {
+    // the single-wave window kernel derives delta from P and dP
+  } else if (head_dim % vecw == 0 && o_stride % vecw == 0 && do_stride % vecw == 0 && part_bytes <= 48 * 1024 && mvit_aligned16(o) && mvit_aligned16(d_o)) {
     const int dgrid = (int)((total + 15) / 16);
     if (dtype == MVIT_BF16)
       hipLaunchKernelGGL((attn_delta_rows_kernel<bf16_t>), dgrid, 256, part_bytes, s, (const bf16_t*)o, (const bf16_t*)d_o, delta, total, nheads, head_dim, o_stride, do_stride);
