@@ -39,6 +39,7 @@ struct GemmParams {
   int64_t k_chunk;    // K extent of one slice (multiple of BK)
   float* workspace;   // [split_k][M][N] fp32 partial sums when split_k > 1
   int vec_ok;         // every epilogue pointer / stride allows 16-byte accesses
+  int flags;          // tuning switches: 2 = one work-group per tile instead of persistent work-groups
   int panel_w;        // tiles are walked in panels of this many tile columns (M fastest across a panel's rows)
 };
 
@@ -376,12 +377,51 @@ __device__ __forceinline__ void emit8(const GemmParams& p, int64_t m, int64_t n,
   else emit8_impl<T, TO, EPI, false>(p, m, n, v, u);
 }
 
+// Per-element epilogue inputs (residual / saved activations) of an interior tile, fetched ahead of their use.
+// One pass of the epilogue covers (BM/WM)*32 rows; a thread owns ITEMS 8-column groups per pass.  Two passes are
+// buffered (one when an element needs two inputs): the epilogue requests pass a+2 when pass a has been consumed.
+template <typename T, int EPI, int BM, int BN, int WM, int NTHREADS>
+struct EpiPre {
+  static constexpr bool DUAL = (EPI == MVIT_EPI_SWIGLU);
+  static constexpr int PASS_ROWS = (BM / WM) * 32, GROUPS = (DUAL ? BN / 2 : BN) / 8;
+  static constexpr bool HAS_IN = (EPI == MVIT_EPI_BIAS_RES || EPI == MVIT_EPI_GELU_BWD || EPI == MVIT_EPI_SWIGLU_BWD) &&
+                                 (PASS_ROWS * GROUPS) % NTHREADS == 0;
+  static constexpr int ITEMS = HAS_IN ? PASS_ROWS * GROUPS / NTHREADS : 1, NLOAD = EPI == MVIT_EPI_SWIGLU_BWD ? 2 : 1;
+  static constexpr int RPI = NTHREADS / GROUPS;  // rows between a thread's consecutive items
+  static_assert(!HAS_IN || (NTHREADS % GROUPS == 0 && 32 % RPI == 0), "row mapping of the prefetched epilogue");
+  typedef T raw8 __attribute__((ext_vector_type(8)));
+  static constexpr int NBUF = NLOAD == 2 ? 1 : 2;  // passes buffered (two 16-byte inputs per element: one pass)
+  raw8 pre[NBUF][ITEMS][NLOAD];
+  const char* base;     // R + m0 * ldr + n0 (block-uniform)
+  unsigned thread_off;  // this thread's byte offset inside a pass: row threadIdx / GROUPS, column group threadIdx % GROUPS
+  bool active;          // block-uniform: this tile takes the prefetched path
+
+  __device__ __forceinline__ void init(const GemmParams& p, int64_t m0, int64_t n0) {
+    active = HAS_IN && p.vec_ok && m0 + BM <= p.M && n0 + GROUPS * 8 <= p.N && p.ldr * (int64_t)BM * sizeof(T) < (1ll << 31);
+    base = reinterpret_cast<const char*>(static_cast<const T*>(p.R) + m0 * p.ldr + n0);
+    thread_off = (unsigned)(((threadIdx.x / GROUPS) * p.ldr + (threadIdx.x % GROUPS) * 8) * sizeof(T));
+  }
+  // Item `it` of pass a is tile row (RPI*it/32)*WM + a*32 + (RPI*it)%32 + threadIdx/GROUPS: a uniform row offset
+  // (scalar address arithmetic) plus the per-thread offset.
+  template <int BUF>
+  __device__ __forceinline__ void fetch(const GemmParams& p, int a) {
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int rowoff = (RPI * it / 32) * WM + a * 32 + (RPI * it) % 32;
+      const char* r = base + (int64_t)rowoff * p.ldr * (int64_t)sizeof(T);
+      pre[BUF][it][0] = *reinterpret_cast<const raw8*>(r + thread_off);
+      if (NLOAD == 2) pre[BUF][it][1] = *reinterpret_cast<const raw8*>(r + p.aux_off * (int64_t)sizeof(T) + thread_off);
+    }
+  }
+};
+
 // Epilogue shared by every main loop.  acc[a][b][4*j+i] is C[m0 + wm*WM + a*32 + 8*j + 4*(l/32) + i][wave column
 // b*32 + l%32].  Pass a: every wave parks its a-th 32-row sub-tile in LDS (fp32, [(BM/WM)*32 rows][BN + 8]), then
 // the block walks the pass in 8-column groups.  The caller guarantees that no wave still reads operands from LDS.
 template <typename T, typename TO, int EPI, int BM, int BN, int WM, int WN, int NTHREADS>
 __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[WM / 32][WN / 32], unsigned char* smem_raw,
-                                             int64_t m0, int64_t n0, int wm, int wn, int slice) {
+                                             int64_t m0, int64_t n0, int wm, int wn, int slice,
+                                             EpiPre<T, EPI, BM, BN, WM, NTHREADS>& ep) {
   constexpr int MT = WM / 32, NT = WN / 32;
   constexpr bool DUAL = (EPI == MVIT_EPI_SWIGLU);
   const int l = threadIdx.x & 63;
@@ -395,25 +435,15 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
   float* ws = to_ws ? p.workspace + (int64_t)slice * p.M * p.N : nullptr;
   const bool ws_vec = (p.N % 4 == 0);
 
-  // Tiles inside the matrix whose epilogue reads one value per output element: those reads are issued one pass
-  // ahead, so their latency hides behind the LDS staging and the previous pass's arithmetic and stores.
-  constexpr bool HAS_IN = (EPI == MVIT_EPI_BIAS_RES || EPI == MVIT_EPI_GELU_BWD || EPI == MVIT_EPI_SWIGLU_BWD);
-  if constexpr (HAS_IN && (PASS_ROWS * GROUPS) % NTHREADS == 0) {
-    if (p.vec_ok && m0 + BM <= p.M && n0 + NCOLS <= p.N) {
-      constexpr int ITEMS = PASS_ROWS * GROUPS / NTHREADS, NLOAD = EPI == MVIT_EPI_SWIGLU_BWD ? 2 : 1;
-      typedef T raw8 __attribute__((ext_vector_type(8)));
-      const T* Rp = static_cast<const T*>(p.R);
-      raw8 pre[2][ITEMS][NLOAD];
-      auto fetch = [&](int a, raw8(&dst)[ITEMS][NLOAD]) {
-#pragma unroll
-        for (int it = 0; it < ITEMS; ++it) {
-          const int c = threadIdx.x + NTHREADS * it, row = c / GROUPS, cg = c % GROUPS;
-          const T* r = Rp + (m0 + (row / 32) * WM + a * 32 + (row % 32)) * p.ldr + n0 + cg * 8;
-          dst[it][0] = *reinterpret_cast<const raw8*>(r);
-          if (NLOAD == 2) dst[it][1] = *reinterpret_cast<const raw8*>(r + p.aux_off);
-        }
-      };
-      fetch(0, pre[0]);
+  // Tiles inside the matrix whose epilogue reads one value per output element: those reads run up to two passes
+  // ahead, so their latency hides behind the LDS staging and the previous passes' arithmetic and stores.
+  using EP = EpiPre<T, EPI, BM, BN, WM, NTHREADS>;
+  if constexpr (EP::HAS_IN) {
+    if (ep.active) {
+      constexpr int ITEMS = EP::ITEMS;
+      constexpr int NBUF = EP::NBUF;
+      ep.template fetch<0>(p, 0);
+      if (NBUF == 2 && MT > 1) ep.template fetch<(NBUF - 1)>(p, 1);
 #pragma unroll
       for (int a = 0; a < MT; ++a) {
         if (a > 0) __syncthreads();
@@ -426,14 +456,17 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
             for (int i = 0; i < 4; ++i) stage[(wm * 32 + 8 * j + lr + i) * SP + col] = acc[a][b][4 * j + i];
         }
         __syncthreads();
-        if (a + 1 < MT) fetch(a + 1, pre[(a + 1) & 1]);
 #pragma unroll
         for (int it = 0; it < ITEMS; ++it) {
           const int c = threadIdx.x + NTHREADS * it, row = c / GROUPS, cg = c % GROUPS;
           const float* sp = stage + row * SP + cg * 8;
           const f32x4 v0 = *reinterpret_cast<const f32x4*>(sp), v1 = *reinterpret_cast<const f32x4*>(sp + 4);
           float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-          emit8_impl<T, TO, EPI, true, true>(p, m0 + (row / 32) * WM + a * 32 + (row % 32), n0 + cg * 8, v, nullptr, pre[a & 1][it]);
+          emit8_impl<T, TO, EPI, true, true>(p, m0 + (row / 32) * WM + a * 32 + (row % 32), n0 + cg * 8, v, nullptr, ep.pre[a % NBUF][it]);
+        }
+        if (a + NBUF < MT) {
+          if ((a % NBUF) == 1) ep.template fetch<(NBUF - 1)>(p, a + NBUF);
+          else ep.template fetch<0>(p, a + NBUF);
         }
       }
       return;
@@ -608,7 +641,9 @@ __global__ __launch_bounds__(Waves<VAR>::NTHREADS, Waves<VAR>::MIN_WAVES) void g
   }
   if (STAGES == 1) __syncthreads();  // operands fully consumed before LDS is reused for the epilogue
 
-  run_epilogue<T, TO, EPI, BM, BN, WM, WN, NTHREADS>(p, acc, smem_raw, m0, n0, wm, wn, slice);
+  EpiPre<T, EPI, BM, BN, WM, NTHREADS> ep;
+  ep.init(p, m0, n0);
+  run_epilogue<T, TO, EPI, BM, BN, WM, WN, NTHREADS>(p, acc, smem_raw, m0, n0, wm, wn, slice, ep);
 }
 
 // ---- bf16 main loop with direct global -> LDS loads (no staging registers) ----------------------------------
@@ -757,8 +792,20 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
   const int tiles = p.tiles_m * p.tiles_n;
   const int total = tiles * p.split_k;
   const int per_xcd = (total + 7) / 8;
-  const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (work >= total) return;
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wv / WGN, wn = wv % WGN;
+  DlFrag<TA, MT> ra;
+  DlFrag<TB, NT> rb;
+  ra.init(wm * WM, 0);
+  rb.init(wn * WN, NSTAGE * TILE);
+  typedef __attribute__((address_space(3))) unsigned char lds_byte;
+  const unsigned lds0 = (unsigned)(__UINTPTR_TYPE__)(lds_byte*)smem_raw + wv * SLICE;
+
+  // Persistent work-groups: the grid has at most one work-group per CU; work-group (xcd, slot) walks that XCD's
+  // tile range with stride slots-per-XCD, the order a one-tile-per-work-group grid would be dispatched in.
+  for (int idx = blockIdx.x >> 3; idx < per_xcd; idx += gridDim.x >> 3) {
+  const int work = (blockIdx.x & 7) * per_xcd + idx;
+  if (work >= total) break;
   const int slice = work / tiles, tile = work % tiles;
   int tm, tn;
   tile_coords(p, tile, tm, tn);
@@ -766,9 +813,6 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
   const int64_t k_end = p.split_k > 1 ? (k_begin + p.k_chunk < p.K ? k_begin + p.k_chunk : p.K) : p.K;
   constexpr int N_PER_BLOCK = DUAL ? BN / 2 : BN;
   const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * N_PER_BLOCK;
-
-  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int wm = wv / WGN, wn = wv % WGN;
 
   f32x16 acc[MT][NT];
 #pragma unroll
@@ -778,20 +822,14 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
+  EpiPre<T, EPI, BM, BN, WM, D::NTHREADS> ep;
+  ep.init(p, m0, n0);
   DlOperand<TA, false, NW> la;
   DlOperand<TB, DUAL, NW> lb;
   la.init(static_cast<const T*>(p.A), nullptr, p.lda, m0, p.M, k_begin, wv);
   lb.init(static_cast<const T*>(p.B), static_cast<const T*>(p.B2), p.ldb, n0, p.N, k_begin, wv);
-  DlFrag<TA, MT> ra;
-  DlFrag<TB, NT> rb;
-  ra.init(wm * WM, 0);
-  rb.init(wn * WN, NSTAGE * TILE);
-
   const int klen = (int)(k_end - k_begin);
   const int T_ = (klen + DL_BK - 1) / DL_BK, k_tail = klen % DL_BK;
-  typedef __attribute__((address_space(3))) unsigned char lds_byte;
-  const unsigned lds0 = (unsigned)(__UINTPTR_TYPE__)(lds_byte*)smem_raw + wv * SLICE;
-
   auto issue = [&](int t, int s) {  // K tile t into stage s (both wave-uniform)
     if (t >= T_) return;
     if (k_tail != 0 && t == T_ - 1) {
@@ -860,7 +898,9 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
     }
   }
   __syncthreads();  // operands fully consumed before LDS is reused by the epilogue
-  run_epilogue<T, TO, EPI, BM, BN, WM, WN, D::NTHREADS>(p, acc, smem_raw, m0, n0, wm, wn, slice);
+  run_epilogue<T, TO, EPI, BM, BN, WM, WN, D::NTHREADS>(p, acc, smem_raw, m0, n0, wm, wn, slice, ep);
+  __syncthreads();  // the staging area is free again before the next tile's operands land in it
+  }
 }
 
 // C[m, n] = sum over slices of the fp32 partial tiles (fixed order, so the result is reproducible).
@@ -920,7 +960,14 @@ int launch_dl(const GemmParams& p, hipStream_t stream) {
   }
   if (p.split_k > 1 && EPI != MVIT_EPI_NONE) return mvit_set_error(MVIT_ERR_UNSUPPORTED, "gemm: split_k needs EPI_NONE");
   const int total = p.tiles_m * p.tiles_n * p.split_k;
-  const int grid = ((total + 7) / 8) * 8;
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+    n_cu = v / 8 * 8 > 0 ? v / 8 * 8 : 8;
+  }
+  const int want = ((total + 7) / 8) * 8;
+  const int grid = (want < n_cu || (p.flags & 2)) ? want : n_cu;
   hipLaunchKernelGGL(kern, grid, D::NTHREADS, lds, stream, p);
   MVIT_CHECK_LAUNCH("gemm");
   if (p.split_k > 1) {
@@ -1022,7 +1069,8 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
   MVIT_REQUIRE(tm * tn < (1ll << 30), "gemm: too many tiles");
   p.tiles_m = (int)tm; p.tiles_n = (int)tn;
   p.panel_w = tn <= 6 ? (int)tn : 4;
-  if (a->reserved2 > 0) p.panel_w = a->reserved2 < tn ? a->reserved2 : (int)tn;  // tuning override
+  p.flags = (a->reserved2 >> 8) & 0xff;
+  if ((a->reserved2 & 0xff) > 0) p.panel_w = (a->reserved2 & 0xff) < tn ? (a->reserved2 & 0xff) : (int)tn;  // tuning override
   p.split_k = 1; p.k_chunk = a->K; p.workspace = nullptr;
   if (a->split_k > 1) {
     const int bk = a->dtype == MVIT_BF16 ? 64 : 16;
