@@ -177,6 +177,34 @@ struct TileStager {
   }
 };
 
+// Reductions over the four lanes l, l^16, l^32, l^48 (the lanes that share one query / key column) with the
+// VALU lane-swap instructions of gfx950 instead of LDS permutes: v_permlane32_swap exchanges the upper half of its
+// first operand with the lower half of its second, v_permlane16_swap does the same for the odd / even rows of 16.
+__device__ __forceinline__ float quad_max(float x) {
+  float a = x, b = x;
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  x = fmaxf(a, b);
+  a = x;
+  b = x;
+  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  return fmaxf(a, b);
+}
+
+// dot_frag with one extra contraction slot (odd ND only: the 16-wide remainder leaves half of its 32-wide MFMA
+// empty): adds a_x * b_x from lane group 0, which is how the forward folds "- running maximum" into the scores.
+template <int ND>
+__device__ __forceinline__ f32x4 dot_frag_plus(const RowFrag<ND>& a, const RowFrag<ND>& b, bf16_t a_x, bf16_t b_x) {
+  using G = Geo<ND>;
+  static_assert(G::TAIL16, "needs the spare slots of the padded remainder");
+  f32x4 c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int ks = 0; ks < G::NK32; ++ks) c = mfma32(a.k32[ks], b.k32[ks], c);
+  const bf16_t z = (bf16_t)0.f;
+  const bf16x8 ax = {a.k16[0], a.k16[1], a.k16[2], a.k16[3], a_x, z, z, z};
+  const bf16x8 bx = {b.k16[0], b.k16[1], b.k16[2], b.k16[3], b_x, z, z, z};
+  return mfma32(ax, bx, c);
+}
+
 __device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
 
 // ================================================================================================
@@ -202,23 +230,42 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void attn_fwd_mfma(const AttnParams
   const bf16_t* K = static_cast<const bf16_t*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD;
   const bf16_t* V = static_cast<const bf16_t*>(p.v) + (int64_t)s0 * p.v_stride + (int64_t)h * HD;
 
+  // Q is scaled by softmax_scale * log2(e) once (rounded to bf16), so the MFMA hands out scores in log2 units.
+  // With an odd ND the spare contraction slot of the padded remainder also subtracts the row's running
+  // stabiliser m_run (kept as a bf16-representable number): exp2 is then applied to the MFMA result directly.
+  constexpr bool FOLD = G::TAIL16;
+  constexpr float TAU = 2.f;  // the stabiliser only moves when a score exceeds it by more than TAU (log2 units)
+  const float c = p.scale * LOG2E;
   RowFrag<ND> qf[4];
 #pragma unroll
   for (int qb = 0; qb < 4; ++qb) {
     const int qi = q0 + qb * 16 + r;
     load_rowfrag_global<ND>(qf[qb], Q + (int64_t)qi * p.q_stride, qi < L, g);
+#pragma unroll
+    for (int ks = 0; ks < G::NK32; ++ks)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) qf[qb].k32[ks][j] = (bf16_t)((float)qf[qb].k32[ks][j] * c);
+    if (G::TAIL16) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) qf[qb].k16[j] = (bf16_t)((float)qf[qb].k16[j] * c);
+    }
   }
+  const bf16_t one_x = (bf16_t)(g == 0 ? 1.f : 0.f);  // key side of the extra slot
+  bf16_t negm_x[4];                                    // query side: -m_run in lane group 0
 
-  f32x4 o[4][ND];
-  float m_run[4], l_run[4];
+  f32x4 o[4][ND], lacc[4];  // lacc: row sums of P, accumulated by the MFMA against a tile of ones
+  float m_run[4];
 #pragma unroll
   for (int qb = 0; qb < 4; ++qb) {
-    m_run[qb] = -INFINITY;
-    l_run[qb] = 0.f;
+    m_run[qb] = 0.f;
+    negm_x[qb] = (bf16_t)0.f;
+    lacc[qb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int dt = 0; dt < ND; ++dt) o[qb][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
-  const float c = p.scale * LOG2E;
+  bf16x8 ones;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) ones[j] = (bf16_t)1.f;
 
   TileStager<ND, BNK, G::PK, PIPE ? NT : BNK * G::CH> sk;  // (degenerate when not pipelined)
   TileStager<ND, BNK, G::PV, PIPE ? NT : BNK * G::CH> sv;
@@ -258,7 +305,10 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void attn_fwd_mfma(const AttnParams
       RowFrag<ND> kf;
       load_rowfrag_lds<ND, G::PK>(kf, tk, kt * 16 + r, g);
 #pragma unroll
-      for (int qb = 0; qb < 4; ++qb) s[qb][kt] = dot_frag<ND>(kf, qf[qb]);
+      for (int qb = 0; qb < 4; ++qb) {
+        if constexpr (FOLD) s[qb][kt] = dot_frag_plus<ND>(kf, qf[qb], one_x, negm_x[qb]);  // log2-scaled score - m_run
+        else s[qb][kt] = dot_frag<ND>(kf, qf[qb]);
+      }
     }
     if (valid < BNK) {  // last, partial tile of the segment
 #pragma unroll
@@ -279,27 +329,31 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void attn_fwd_mfma(const AttnParams
         mx = max3(mx, s[qb][kt][0], s[qb][kt][1]);
         mx = max3(mx, s[qb][kt][2], s[qb][kt][3]);
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run[qb], mx * c);  // c > 0; finite: every tile holds at least one valid key
-      if (__builtin_amdgcn_ballot_w64(m_new > m_run[qb]) != 0) {
-        const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_new);
+      mx = quad_max(mx);
+      if (!FOLD) mx -= m_run[qb];  // excess over the current stabiliser
+      const bool grow = k0 == 0 || mx > TAU;
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+        float m_new = grow ? m_run[qb] + mx : m_run[qb];
+        if (FOLD) m_new = (float)(bf16_t)m_new;
+        const float delta = m_new - m_run[qb];
+        const float alpha = k0 == 0 ? 1.f : __builtin_amdgcn_exp2f(-delta);
         m_run[qb] = m_new;
-        l_run[qb] *= alpha;
+        lacc[qb] *= alpha;
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt) o[qb][dt] *= alpha;
+        if (FOLD) {  // this tile's scores were taken against the old stabiliser
+          negm_x[qb] = (bf16_t)(g == 0 ? -m_new : 0.f);
+#pragma unroll
+          for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s[qb][kt][i] -= delta;
+        }
       }
-      const float neg_m = -m_run[qb];
-      float ps = 0.f;
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][kt][i], c, neg_m));
-          s[qb][kt][i] = e;
-          ps += e;
-        }
-      l_run[qb] += ps;
+        for (int i = 0; i < 4; ++i)
+          s[qb][kt][i] = __builtin_amdgcn_exp2f(FOLD ? s[qb][kt][i] : s[qb][kt][i] - m_run[qb]);
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) pb[qb][kk] = pack8(s[qb][2 * kk], s[qb][2 * kk + 1]);
     }
@@ -313,6 +367,10 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void attn_fwd_mfma(const AttnParams
 #pragma unroll
         for (int qb = 0; qb < 4; ++qb) o[qb][dt] = mfma32(vf, pb[qb][kk], o[qb][dt]);
       }
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+      for (int qb = 0; qb < 4; ++qb) lacc[qb] = mfma32(ones, pb[qb][kk], lacc[qb]);
     if (PIPE) {
       if (has_next) {
         sk.store(lds_k[buf ^ 1]);
@@ -326,9 +384,7 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void attn_fwd_mfma(const AttnParams
   bf16_t* O = static_cast<bf16_t*>(p.out) + (int64_t)s0 * p.o_stride + (int64_t)h * HD;
 #pragma unroll
   for (int qb = 0; qb < 4; ++qb) {
-    float lt = l_run[qb];
-    lt += __shfl_xor(lt, 16, 64);
-    lt += __shfl_xor(lt, 32, 64);
+    const float lt = lacc[qb][0];  // every row of the ones tile holds the row sum
     const int qi = q0 + qb * 16 + r;
     if (qi < L) {
       const float inv = 1.f / lt;
