@@ -208,12 +208,12 @@ __device__ __forceinline__ f32x4 dot_frag_plus(const RowFrag<ND>& a, const RowFr
 __device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
 
 // ================================================================================================
-// Forward.  Block = NWAVES waves = 64*NWAVES queries of one (segment, head); 64 keys per iteration.
-// Two work-groups share a CU (<= 256 registers), K/V tiles are double buffered in LDS and the next tile is
+// Forward.  Block = NWAVES waves x 16*QB queries of one (segment, head); BNK keys per iteration.
+// At least two work-groups share a CU, K/V tiles are double buffered in LDS and the next tile is
 // fetched while the current one is used; key masking only runs on a segment's last, partial tile; the output
 // accumulators are rescaled only in iterations where some row maximum of the wave actually grew.
-template <int ND, int NWAVES, int BNK, bool PIPE>
-__global__ __launch_bounds__(64 * NWAVES, 2) void attn_fwd_mfma(const AttnParams p) {
+template <int ND, int NWAVES, int BNK, bool PIPE, int QB = 4, int MINW = 2>
+__global__ __launch_bounds__(64 * NWAVES, MINW) void attn_fwd_mfma(const AttnParams p) {
   using G = Geo<ND>;
   constexpr int HD = G::HD, NT = 64 * NWAVES, KT = BNK / 16, KK = BNK / 32, NBUF = PIPE ? 2 : 1;
   __shared__ __attribute__((aligned(16))) bf16_t lds_k[NBUF][BNK * G::PK];
@@ -221,10 +221,10 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void attn_fwd_mfma(const AttnParams
 
   const int seg = blockIdx.y, h = blockIdx.z;
   const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
-  const int blk_q0 = blockIdx.x * NT;
+  const int blk_q0 = blockIdx.x * (16 * QB * NWAVES);
   if (blk_q0 >= L) return;
   const int l = threadIdx.x & 63, wv = threadIdx.x >> 6, g = l >> 4, r = l & 15;
-  const int q0 = blk_q0 + wv * 64;
+  const int q0 = blk_q0 + wv * (16 * QB);
 
   const bf16_t* Q = static_cast<const bf16_t*>(p.q) + (int64_t)s0 * p.q_stride + (int64_t)h * HD;
   const bf16_t* K = static_cast<const bf16_t*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD;
@@ -236,9 +236,9 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void attn_fwd_mfma(const AttnParams
   constexpr bool FOLD = G::TAIL16;
   constexpr float TAU = 2.f;  // the stabiliser only moves when a score exceeds it by more than TAU (log2 units)
   const float c = p.scale * LOG2E;
-  RowFrag<ND> qf[4];
+  RowFrag<ND> qf[QB];
 #pragma unroll
-  for (int qb = 0; qb < 4; ++qb) {
+  for (int qb = 0; qb < QB; ++qb) {
     const int qi = q0 + qb * 16 + r;
     load_rowfrag_global<ND>(qf[qb], Q + (int64_t)qi * p.q_stride, qi < L, g);
 #pragma unroll
@@ -251,12 +251,12 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void attn_fwd_mfma(const AttnParams
     }
   }
   const bf16_t one_x = (bf16_t)(g == 0 ? 1.f : 0.f);  // key side of the extra slot
-  bf16_t negm_x[4];                                    // query side: -m_run in lane group 0
+  bf16_t negm_x[QB];                                    // query side: -m_run in lane group 0
 
-  f32x4 o[4][ND], lacc[4];  // lacc: row sums of P, accumulated by the MFMA against a tile of ones
-  float m_run[4];
+  f32x4 o[QB][ND], lacc[QB];  // lacc: row sums of P, accumulated by the MFMA against a tile of ones
+  float m_run[QB];
 #pragma unroll
-  for (int qb = 0; qb < 4; ++qb) {
+  for (int qb = 0; qb < QB; ++qb) {
     m_run[qb] = 0.f;
     negm_x[qb] = (bf16_t)0.f;
     lacc[qb] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -299,29 +299,29 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void attn_fwd_mfma(const AttnParams
     const bf16_t* tv = lds_v[PIPE ? buf : 0];
 
     // raw scores: s[qb][kt][i] = S[query qb*16 + r][key kt*16 + 4g + i]
-    f32x4 s[4][KT];
+    f32x4 s[QB][KT];
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
       RowFrag<ND> kf;
       load_rowfrag_lds<ND, G::PK>(kf, tk, kt * 16 + r, g);
 #pragma unroll
-      for (int qb = 0; qb < 4; ++qb) {
+      for (int qb = 0; qb < QB; ++qb) {
         if constexpr (FOLD) s[qb][kt] = dot_frag_plus<ND>(kf, qf[qb], one_x, negm_x[qb]);  // log2-scaled score - m_run
         else s[qb][kt] = dot_frag<ND>(kf, qf[qb]);
       }
     }
     if (valid < BNK) {  // last, partial tile of the segment
 #pragma unroll
-      for (int qb = 0; qb < 4; ++qb)
+      for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
           for (int i = 0; i < 4; ++i)
             if (kt * 16 + 4 * g + i >= valid) s[qb][kt][i] = -INFINITY;
     }
-    bf16x8 pb[4][KK];
+    bf16x8 pb[QB][KK];
 #pragma unroll
-    for (int qb = 0; qb < 4; ++qb) {
+    for (int qb = 0; qb < QB; ++qb) {
       float mx = fmaxf(s[qb][0][0], s[qb][0][1]);
       mx = max3(mx, s[qb][0][2], s[qb][0][3]);
 #pragma unroll
@@ -365,12 +365,12 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void attn_fwd_mfma(const AttnParams
         const bf16_t* a0 = tv + ((2 * kk) * 16 + 4 * g + (r >> 2)) * G::PV + 16 * dt + 4 * (r & 3);
         const bf16x8 vf = tr_pair(a0, a0 + 16 * G::PV);
 #pragma unroll
-        for (int qb = 0; qb < 4; ++qb) o[qb][dt] = mfma32(vf, pb[qb][kk], o[qb][dt]);
+        for (int qb = 0; qb < QB; ++qb) o[qb][dt] = mfma32(vf, pb[qb][kk], o[qb][dt]);
       }
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
-      for (int qb = 0; qb < 4; ++qb) lacc[qb] = mfma32(ones, pb[qb][kk], lacc[qb]);
+      for (int qb = 0; qb < QB; ++qb) lacc[qb] = mfma32(ones, pb[qb][kk], lacc[qb]);
     if (PIPE) {
       if (has_next) {
         sk.store(lds_k[buf ^ 1]);
@@ -383,7 +383,7 @@ __global__ __launch_bounds__(64 * NWAVES, 2) void attn_fwd_mfma(const AttnParams
 
   bf16_t* O = static_cast<bf16_t*>(p.out) + (int64_t)s0 * p.o_stride + (int64_t)h * HD;
 #pragma unroll
-  for (int qb = 0; qb < 4; ++qb) {
+  for (int qb = 0; qb < QB; ++qb) {
     const float lt = lacc[qb][0];  // every row of the ones tile holds the row sum
     const int qi = q0 + qb * 16 + r;
     if (qi < L) {
@@ -1118,7 +1118,12 @@ int launch_fwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
   dim3 grid((unsigned)((max_seqlen + 64 * nw - 1) / (64 * nw)), (unsigned)n_seg, (unsigned)p.nheads);
   if (nw == 1) hipLaunchKernelGGL((attn_fwd_mfma<ND, 1, 64, false>), grid, 64, 0, s, p);
   else if (nw == 2) hipLaunchKernelGGL((attn_fwd_mfma<ND, 2, 64, false>), grid, 128, 0, s, p);
-  else hipLaunchKernelGGL((attn_fwd_mfma<ND, 4, 32, true>), grid, 256, 0, s, p);
+  else if constexpr (ND <= 5) {
+    // long segments: 8 waves x 32 queries, <= 128 registers, so that four waves share a SIMD and cover each
+    // other's MFMA -> softmax -> MFMA dependency stalls
+    hipLaunchKernelGGL((attn_fwd_mfma<ND, 8, 32, true, 2, 4>), grid, 512, 0, s, p);
+  }
+  else hipLaunchKernelGGL((attn_fwd_mfma<ND, 4, 32, true>), grid, 256, 0, s, p);  // head_dim 128: register budget
   MVIT_CHECK_LAUNCH("attn_fwd");
   return MVIT_OK;
 }
