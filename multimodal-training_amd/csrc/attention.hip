@@ -63,6 +63,30 @@ struct Geo {
   static constexpr int CH = 2 * ND;           // 16-byte chunks per row
 };
 
+// Bank-rotated LDS tile layout for tiles that are read both row-wise (16-byte fragments of 16 consecutive rows)
+// and through the transposing load (8 consecutive rows x 32 bytes): chunk c (16 bytes) of row r lives at byte
+// r * 512 + 16 * (c + rot(r)), rot(r) = 2 * (r & 7) + ((r >> 3) & 1).  Modulo the 256 bytes of one pass over the
+// banks, sixteen consecutive rows put one chunk index into sixteen different 16-byte slots, and eight consecutive
+// rows put one pair of chunks into eight disjoint 32-byte windows, so neither access pattern has bank conflicts
+// (a plain pitch cannot satisfy both: the first needs pitch/16 odd, the second pitch/32 odd).  The rotation is
+// additive, so every access is a per-lane base plus a compile-time offset; rows are 512 bytes so that it never
+// wraps (10 chunks of data + rotation <= 25 slots; head_dim 128: 31).
+constexpr int SWZ = 256;  // pitch in elements; used as the PITCH argument to select this layout
+__device__ __forceinline__ int swz_off(int row, int chunk) {
+  return row * SWZ + ((chunk + (((row & 7) << 1) | ((row >> 3) & 1))) << 3);
+}
+// Transposed operand of the 16 x 16 block (rows row0.., head-dim 16*d..) : two transposing loads 16 rows apart.
+template <int PITCH>
+__device__ __forceinline__ bf16x8 tr_block(const bf16_t* tile, int row0, int d, int g, int r) {
+  const int row = row0 + 4 * g + (r >> 2);
+  if (PITCH == SWZ) {
+    const int chunk = 2 * d + ((r & 3) >> 1), sub = 4 * (r & 1);
+    return tr_pair(tile + swz_off(row, chunk) + sub, tile + swz_off(row + 16, chunk) + sub);
+  }
+  const bf16_t* a = tile + row * PITCH + 16 * d + 4 * (r & 3);
+  return tr_pair(a, a + 16 * PITCH);
+}
+
 // Operand fragments of 16 rows x head_dim for one lane, in the "row l%16, contraction 8*(l/16)+j" layout
 // (serves as MFMA A for rows, or as MFMA B for columns).
 template <int ND>
@@ -91,6 +115,12 @@ __device__ __forceinline__ void load_rowfrag_global(RowFrag<ND>& f, const bf16_t
 template <int ND, int PITCH>
 __device__ __forceinline__ void load_rowfrag_lds(RowFrag<ND>& f, const bf16_t* tile, int row, int g) {
   using G = Geo<ND>;
+  if (PITCH == SWZ) {
+#pragma unroll
+    for (int ks = 0; ks < G::NK32; ++ks) f.k32[ks] = *reinterpret_cast<const bf16x8*>(tile + swz_off(row, 4 * ks + g));
+    if (G::TAIL16) f.k16 = *reinterpret_cast<const bf16x4*>(tile + swz_off(row, 4 * G::NK32 + (g >> 1)) + 4 * (g & 1));
+    return;
+  }
   const bf16_t* p = tile + row * PITCH;
 #pragma unroll
   for (int ks = 0; ks < G::NK32; ++ks) f.k32[ks] = *reinterpret_cast<const bf16x8*>(p + 32 * ks + 8 * g);
@@ -156,7 +186,7 @@ struct TileStager {
       const int c = threadIdx.x + NTHREADS * i;
       const int r = c / G::CH, dc = c % G::CH;
       row[i] = c < CHUNKS ? r : ROWS;
-      lds_off[i] = r * PITCH + dc * 8;
+      lds_off[i] = PITCH == SWZ ? swz_off(r, dc) : r * PITCH + dc * 8;
       goff[i] = (int64_t)r * stride + dc * 8;
     }
   }
@@ -169,6 +199,12 @@ struct TileStager {
       if (row[i] < valid_rows) v = *reinterpret_cast<const bf16x8*>(src + goff[i]);
       regs[i] = v;
     }
+  }
+  __device__ __forceinline__ void scale(float c) {  // the loaded chunks times c, rounded back to bf16
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) regs[i][j] = (bf16_t)((float)regs[i][j] * c);
   }
   __device__ __forceinline__ void store(bf16_t* tile) const {
 #pragma unroll
@@ -203,6 +239,44 @@ __device__ __forceinline__ f32x4 dot_frag_plus(const RowFrag<ND>& a, const RowFr
   const bf16x8 ax = {a.k16[0], a.k16[1], a.k16[2], a.k16[3], a_x, z, z, z};
   const bf16x8 bx = {b.k16[0], b.k16[1], b.k16[2], b.k16[3], b_x, z, z, z};
   return mfma32(ax, bx, c);
+}
+
+// A float as the sum of two bf16 numbers (16 bits of mantissa): for values that ride in spare contraction slots.
+struct HiLo {
+  bf16_t hi, lo;
+};
+__device__ __forceinline__ HiLo split_hilo(float x) {
+  HiLo r;
+  r.hi = (bf16_t)x;
+  r.lo = (bf16_t)(x - (float)r.hi);
+  return r;
+}
+// dot_frag with two extra contraction slots: adds a0*b0 + a1*b1 (operands given per lane; lane groups other than
+// 0 must pass zeros on at least one side).  The backward uses it for "- lse" and "- delta", split as hi + lo.
+template <int ND>
+__device__ __forceinline__ f32x4 dot_frag_plus2(const RowFrag<ND>& a, const RowFrag<ND>& b, bf16_t a0, bf16_t a1, bf16_t b0, bf16_t b1) {
+  using G = Geo<ND>;
+  static_assert(G::TAIL16, "needs the spare slots of the padded remainder");
+  f32x4 c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int ks = 0; ks < G::NK32; ++ks) c = mfma32(a.k32[ks], b.k32[ks], c);
+  const bf16_t z = (bf16_t)0.f;
+  const bf16x8 ax = {a.k16[0], a.k16[1], a.k16[2], a.k16[3], a0, a1, z, z};
+  const bf16x8 bx = {b.k16[0], b.k16[1], b.k16[2], b.k16[3], b0, b1, z, z};
+  return mfma32(ax, bx, c);
+}
+// Multiply a fragment by a scalar (rounded back to bf16): Q enters every score product as Q * scale * log2(e).
+template <int ND>
+__device__ __forceinline__ void scale_rowfrag(RowFrag<ND>& f, float c) {
+  using G = Geo<ND>;
+#pragma unroll
+  for (int ks = 0; ks < G::NK32; ++ks)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f.k32[ks][j] = (bf16_t)((float)f.k32[ks][j] * c);
+  if (G::TAIL16) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) f.k16[j] = (bf16_t)((float)f.k16[j] * c);
+  }
 }
 
 __device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
@@ -241,14 +315,7 @@ __global__ __launch_bounds__(64 * NWAVES, MINW) void attn_fwd_mfma(const AttnPar
   for (int qb = 0; qb < QB; ++qb) {
     const int qi = q0 + qb * 16 + r;
     load_rowfrag_global<ND>(qf[qb], Q + (int64_t)qi * p.q_stride, qi < L, g);
-#pragma unroll
-    for (int ks = 0; ks < G::NK32; ++ks)
-#pragma unroll
-      for (int j = 0; j < 8; ++j) qf[qb].k32[ks][j] = (bf16_t)((float)qf[qb].k32[ks][j] * c);
-    if (G::TAIL16) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) qf[qb].k16[j] = (bf16_t)((float)qf[qb].k16[j] * c);
-    }
+    scale_rowfrag<ND>(qf[qb], c);
   }
   const bf16_t one_x = (bf16_t)(g == 0 ? 1.f : 0.f);  // key side of the extra slot
   bf16_t negm_x[QB];                                    // query side: -m_run in lane group 0
@@ -468,10 +535,13 @@ template <int ND, int NWAVES, int RB>
 __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnParams p) {
   using G = Geo<ND>;
   constexpr int HD = G::HD, BQ = 32, NT = 64 * NWAVES, SPAN = 16 * RB * NWAVES;  // RB 16-row blocks per wave
-  __shared__ __attribute__((aligned(16))) bf16_t lds_q[2][BQ * G::PK];
-  __shared__ __attribute__((aligned(16))) bf16_t lds_do[2][BQ * G::PK];
+  constexpr int P = SWZ;  // Q / dO tiles are read as row fragments and through the transposing load
+  __shared__ __attribute__((aligned(16))) bf16_t lds_q[2][BQ * P];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_do[2][BQ * P];
   __shared__ __attribute__((aligned(16))) float lds_lse[2][BQ];
   __shared__ __attribute__((aligned(16))) float lds_delta[2][BQ];
+  __shared__ __attribute__((aligned(8))) bf16_t lds_fold[2][BQ][4];  // -lse2 and -delta per row, each as hi + lo
+  constexpr bool FOLD = G::TAIL16;
 
   const int seg = blockIdx.y, h = blockIdx.z;
   const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
@@ -503,15 +573,16 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
       dv[kb][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
   const float c = p.scale * LOG2E;
+  const bf16_t one_x = (bf16_t)(g == 0 ? 1.f : 0.f);
 
-  TileStager<ND, BQ, G::PK, NT> sq, sdo;
+  TileStager<ND, BQ, P, NT> sq, sdo;
   sq.init(p.q_stride);
   sdo.init(p.do_stride);
   float r_lse = 0.f, r_delta = 0.f;  // threads 0..31 carry one row's statistics
   auto load_stats = [&](int qs, int valid) {
     if (threadIdx.x < BQ) {
       const bool ok = (int)threadIdx.x < valid;
-      r_lse = ok ? LSE[qs + threadIdx.x] * LOG2E : INFINITY;  // +inf => p = 0 for padded queries
+      r_lse = ok ? LSE[qs + threadIdx.x] * LOG2E : 1e30f;  // huge => p = 0 for padded queries
       r_delta = ok ? DELTA[qs + threadIdx.x] : 0.f;
     }
   };
@@ -519,11 +590,17 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
     if (threadIdx.x < BQ) {
       lds_lse[b][threadIdx.x] = r_lse;
       lds_delta[b][threadIdx.x] = r_delta;
+      const HiLo nl = split_hilo(-r_lse), nd = split_hilo(-r_delta);
+      lds_fold[b][threadIdx.x][0] = nl.hi;
+      lds_fold[b][threadIdx.x][1] = nl.lo;
+      lds_fold[b][threadIdx.x][2] = nd.hi;
+      lds_fold[b][threadIdx.x][3] = nd.lo;
     }
   };
   sq.load(Q, min(BQ, L));
   sdo.load(DO, min(BQ, L));
   load_stats(0, min(BQ, L));
+  sq.scale(c);  // the Q tile holds Q * scale * log2(e): scores leave the MFMA in log2 units
   sq.store(lds_q[0]);
   sdo.store(lds_do[0]);
   store_stats(0);
@@ -544,31 +621,48 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
     RowFrag<ND> qa[2], da[2];  // natural-layout A operands: row = query t*16 + r
     bf16x8 qt[ND], dt_[ND];    // transposed A operands: row = head-dim 16*dt + r, slots = queries
     f32x4 lse2[2], dl[2];
+    bf16x4 fold[2];  // FOLD: (-lse2 hi, lo, -delta hi, lo) of query t*16 + r, riding in the padded MFMA's spare slots
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      load_rowfrag_lds<ND, G::PK>(qa[t], tq, t * 16 + r, g);
-      load_rowfrag_lds<ND, G::PK>(da[t], tdo, t * 16 + r, g);
-      lse2[t] = *reinterpret_cast<const f32x4*>(lds_lse[buf] + t * 16 + 4 * g);
-      dl[t] = *reinterpret_cast<const f32x4*>(lds_delta[buf] + t * 16 + 4 * g);
+      load_rowfrag_lds<ND, P>(qa[t], tq, t * 16 + r, g);
+      load_rowfrag_lds<ND, P>(da[t], tdo, t * 16 + r, g);
+      if (FOLD) {
+        fold[t] = *reinterpret_cast<const bf16x4*>(lds_fold[buf][t * 16 + r]);
+        if (g != 0) fold[t] = bf16x4{(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
+      } else {
+        lse2[t] = *reinterpret_cast<const f32x4*>(lds_lse[buf] + t * 16 + 4 * g);
+        dl[t] = *reinterpret_cast<const f32x4*>(lds_delta[buf] + t * 16 + 4 * g);
+      }
     }
 #pragma unroll
     for (int d = 0; d < ND; ++d) {
-      const int off = (4 * g + (r >> 2)) * G::PK + 16 * d + 4 * (r & 3);
-      qt[d] = tr_pair(tq + off, tq + off + 16 * G::PK);
-      dt_[d] = tr_pair(tdo + off, tdo + off + 16 * G::PK);
+      qt[d] = tr_block<P>(tq, 0, d, g, r);
+      dt_[d] = tr_block<P>(tdo, 0, d, g, r);
     }
 #pragma unroll
     for (int kb = 0; kb < RB; ++kb) {
       f32x4 pv[2], ds[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        const f32x4 s = dot_frag<ND>(qa[t], kf[kb]);   // S[q = t*16+4g+i][key = kb*16+r]
-        const f32x4 dp = dot_frag<ND>(da[t], vf[kb]);  // dP, same layout
+        // S[q = t*16+4g+i][key = kb*16+r] in log2 units, and dP in the same layout
+        if constexpr (FOLD) {
+          const f32x4 s = dot_frag_plus2<ND>(qa[t], kf[kb], fold[t][0], fold[t][1], one_x, one_x);   // - lse2
+          const f32x4 dp = dot_frag_plus2<ND>(da[t], vf[kb], fold[t][2], fold[t][3], one_x, one_x);  // - delta
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c, -lse2[t][i]));
-          pv[t][i] = e;
-          ds[t][i] = e * (dp[i] - dl[t][i]);
+          for (int i = 0; i < 4; ++i) {
+            const float e = __builtin_amdgcn_exp2f(s[i]);
+            pv[t][i] = e;
+            ds[t][i] = e * dp[i];
+          }
+        } else {
+          const f32x4 s = dot_frag<ND>(qa[t], kf[kb]);
+          const f32x4 dp = dot_frag<ND>(da[t], vf[kb]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float e = __builtin_amdgcn_exp2f(s[i] - lse2[t][i]);
+            pv[t][i] = e;
+            ds[t][i] = e * (dp[i] - dl[t][i]);
+          }
         }
       }
       const bf16x8 pb = pack8(pv[0], pv[1]);
@@ -580,6 +674,7 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
       }
     }
     if (has_next) {
+      sq.scale(c);
       sq.store(lds_q[buf ^ 1]);
       sdo.store(lds_do[buf ^ 1]);
       store_stats(buf ^ 1);
@@ -599,7 +694,7 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
         bf16x4 a, b;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          a[i] = (bf16_t)(dk[kb][d][i] * p.scale);
+          a[i] = (bf16_t)(dk[kb][d][i] * LN2);  // dS^T (Q scale log2e) / log2e
           b[i] = (bf16_t)dv[kb][d][i];
         }
         *reinterpret_cast<bf16x4*>(DK + (int64_t)ki * p.dk_stride + 16 * d + 4 * g) = a;
@@ -615,8 +710,9 @@ template <int ND, int NWAVES, int RB>
 __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams p) {
   using G = Geo<ND>;
   constexpr int HD = G::HD, BK = 32, NT = 64 * NWAVES, SPAN = 16 * RB * NWAVES;  // RB 16-row blocks per wave
-  __shared__ __attribute__((aligned(16))) bf16_t lds_k[2][BK * G::PK];
-  __shared__ __attribute__((aligned(16))) bf16_t lds_v[2][BK * G::PK];
+  constexpr int P = SWZ;  // the K tile is read as row fragments and through the transposing load
+  __shared__ __attribute__((aligned(16))) bf16_t lds_k[2][BK * P];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_v[2][BK * P];
 
   const int seg = blockIdx.y, h = blockIdx.z;
   const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
@@ -632,25 +728,31 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams
   const float* LSE = p.lse + (int64_t)h * p.total + s0;
   const float* DELTA = p.delta + (int64_t)h * p.total + s0;
 
+  constexpr bool FOLD = G::TAIL16;
+  const float c = p.scale * LOG2E;
+  const bf16_t one_x = (bf16_t)(g == 0 ? 1.f : 0.f);
   RowFrag<ND> qf[RB], dof[RB];
   float neg_lse2[RB], dl[RB];
+  HiLo f_lse[RB], f_dl[RB];  // FOLD: -lse2 and -delta of the lane's query as hi + lo (lane group 0 only)
 #pragma unroll
   for (int qb = 0; qb < RB; ++qb) {
     const int qi = q0 + qb * 16 + r;
     const bool ok = qi < L;
     load_rowfrag_global<ND>(qf[qb], Q + (int64_t)qi * p.q_stride, ok, g);
+    scale_rowfrag<ND>(qf[qb], c);  // scores leave the MFMA in log2 units
     load_rowfrag_global<ND>(dof[qb], DO + (int64_t)qi * p.do_stride, ok, g);
-    neg_lse2[qb] = ok ? -LSE[qi] * LOG2E : -INFINITY;
+    neg_lse2[qb] = ok ? -LSE[qi] * LOG2E : -1e30f;  // hugely negative => p = 0 for padded queries
     dl[qb] = ok ? DELTA[qi] : 0.f;
+    f_lse[qb] = split_hilo(g == 0 ? neg_lse2[qb] : 0.f);
+    f_dl[qb] = split_hilo(g == 0 ? -dl[qb] : 0.f);
   }
   f32x4 dq[RB][ND];
 #pragma unroll
   for (int qb = 0; qb < RB; ++qb)
 #pragma unroll
     for (int d = 0; d < ND; ++d) dq[qb][d] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const float c = p.scale * LOG2E;
 
-  TileStager<ND, BK, G::PK, NT> sk, sv;
+  TileStager<ND, BK, P, NT> sk, sv;
   sk.init(p.k_stride);
   sv.init(p.v_stride);
   sk.load(K, min(BK, L));
@@ -675,25 +777,29 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams
     bf16x8 kt[ND];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      load_rowfrag_lds<ND, G::PK>(ka[t], tk, t * 16 + r, g);
-      load_rowfrag_lds<ND, G::PK>(va[t], tv, t * 16 + r, g);
+      load_rowfrag_lds<ND, P>(ka[t], tk, t * 16 + r, g);
+      load_rowfrag_lds<ND, P>(va[t], tv, t * 16 + r, g);
     }
 #pragma unroll
     for (int d = 0; d < ND; ++d) {
-      const int off = (4 * g + (r >> 2)) * G::PK + 16 * d + 4 * (r & 3);
-      kt[d] = tr_pair(tk + off, tk + off + 16 * G::PK);
+      kt[d] = tr_block<P>(tk, 0, d, g, r);
     }
 #pragma unroll
     for (int qb = 0; qb < RB; ++qb) {
       f32x4 ds[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        const f32x4 s = dot_frag<ND>(ka[t], qf[qb]);    // S[q = qb*16+r][key = t*16+4g+i]
-        const f32x4 dp = dot_frag<ND>(va[t], dof[qb]);  // dP, same layout
+        // S[q = qb*16+r][key = t*16+4g+i] in log2 units, and dP in the same layout
+        if constexpr (FOLD) {
+          const f32x4 s = dot_frag_plus2<ND>(ka[t], qf[qb], one_x, one_x, f_lse[qb].hi, f_lse[qb].lo);   // - lse2
+          const f32x4 dp = dot_frag_plus2<ND>(va[t], dof[qb], one_x, one_x, f_dl[qb].hi, f_dl[qb].lo);  // - delta
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], c, neg_lse2[qb]));
-          ds[t][i] = e * (dp[i] - dl[qb]);
+          for (int i = 0; i < 4; ++i) ds[t][i] = __builtin_amdgcn_exp2f(s[i]) * dp[i];
+        } else {
+          const f32x4 s = dot_frag<ND>(ka[t], qf[qb]);
+          const f32x4 dp = dot_frag<ND>(va[t], dof[qb]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) ds[t][i] = __builtin_amdgcn_exp2f(s[i] + neg_lse2[qb]) * (dp[i] - dl[qb]);
         }
       }
       if (valid < BK) {  // keys past the segment end contribute nothing
@@ -764,6 +870,7 @@ __global__ __launch_bounds__(64) void attn_bwd_window_mfma(const AttnParams p) {
     sv.load(static_cast<const bf16_t*>(p.v) + (int64_t)s0 * p.v_stride + (int64_t)h * HD, L);
     sdo.load(static_cast<const bf16_t*>(p.d_o) + (int64_t)s0 * p.do_stride + (int64_t)h * HD, L);
     lds_lse[l] = l < L ? p.lse[(int64_t)h * p.total + s0 + l] * LOG2E : INFINITY;  // +inf => p = 0 for padded queries
+    sq.scale(c);  // the Q tile holds Q * scale * log2(e): scores leave the MFMA in log2 units
     sq.store(lds_q);
     sk.store(lds_k);
     sv.store(lds_v);
@@ -808,7 +915,7 @@ __global__ __launch_bounds__(64) void attn_bwd_window_mfma(const AttnParams p) {
           dp[kc][t] = dot_frag<ND>(va[kc][t], dof);      // dP, same layout
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            float x = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], c, neg_lse2));
+            float x = __builtin_amdgcn_exp2f(sc[i] + neg_lse2);
             if (kc * 32 + t * 16 + 4 * g + i >= L) x = 0.f;  // keys past the segment end
             e[kc][t][i] = x;
             part = __builtin_fmaf(x, dp[kc][t][i], part);
@@ -891,7 +998,7 @@ __global__ __launch_bounds__(64) void attn_bwd_window_mfma(const AttnParams p) {
           const f32x4 dpp = dot_frag<ND>(da[t], vf[kb]);  // dP, same layout
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const float x = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], c, -lse2[t][i]));
+            const float x = __builtin_amdgcn_exp2f(sc[i] - lse2[t][i]);
             pv[t][i] = x;
             ds[t][i] = x * (dpp[i] - dl[t][i]);
           }
@@ -916,7 +1023,7 @@ __global__ __launch_bounds__(64) void attn_bwd_window_mfma(const AttnParams p) {
           bf16x4 a, b;
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            a[i] = (bf16_t)(dk[kb][d][i] * p.scale);
+            a[i] = (bf16_t)(dk[kb][d][i] * LN2);  // dS^T (Q scale log2e) / log2e
             b[i] = (bf16_t)dv[kb][d][i];
           }
           *reinterpret_cast<bf16x4*>(DK + (int64_t)ki * p.dk_stride + 16 * d + 4 * g) = a;
