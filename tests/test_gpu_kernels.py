@@ -142,6 +142,35 @@ def test_split_gather_bit_exact(dtype, sp):
         assert sum(m.total_local_len for m in metas) == S
 
 
+def test_split_gather_sp4_real_shape():
+    """Five square images with sides drawn from the multiples of 28 in [448, 3584] (seed 2), hidden 1280, bf16,
+    split into 4 sequence-parallel shards (token cuts and window-aligned cuts) and gathered back: bit-exact."""
+    from mi355_vit import sequence_parallel_utils as spu
+
+    ops = _ops()
+    g = torch.Generator().manual_seed(2)
+    side = 2 * torch.randint(16, 129, (5,), generator=g)  # patches per side (even: 28 px = 2 patches)
+    grid = torch.stack([torch.ones(5, dtype=torch.long), side, side], dim=1)
+    _, cu_w = ops.window_index(grid, 2, 112, 14)
+    lengths = (side * side).tolist()
+    S = sum(lengths)
+    _announce(f"split/gather real shape: {S} patches")
+    xg = torch.randint(-32768, 32767, (S, 1280), dtype=torch.int16, generator=g).view(torch.bfloat16).to(DEV)
+    x_np = xg.cpu().view(torch.int16).numpy()
+    for windows in (None, cu_w):
+        packs, metas = [], []
+        for r in range(4):
+            pk, meta = spu.split_pack_by_sp(xg, lengths, r, 4, cu_window_seqlens=windows)
+            ref = sp_oracle.split_rows(x_np, lengths, r, 4, None if windows is None else windows.tolist())
+            assert np.array_equal(pk.cpu().view(torch.int16).numpy(), ref)
+            packs.append(pk)
+            metas.append(meta)
+        rebuilt = spu.gather_rank_packs(packs, [m.local_lengths for m in metas])
+        assert torch.equal(rebuilt.view(torch.int16), xg.view(torch.int16))
+        if windows is None:
+            assert max(m.total_local_len for m in metas) - min(m.total_local_len for m in metas) <= len(lengths)
+
+
 def test_split_gather_reference_sizes():
     """tests/test_split_gather.py of the reference: arange tensors of 1024 and 1020 rows x 1280, two ranks."""
     from mi355_vit import sequence_parallel_utils as spu
@@ -362,6 +391,48 @@ def test_attention_long_segment_bf16():
     """One 2,048-token segment with 4 heads (the sequence-parallel share shape, scaled down)."""
     _announce("attention bf16 long")
     _attn_case(torch.bfloat16, [2048, 1000], 4, 80, qkv_packed=False)
+
+
+def test_attention_sp_share_real_shape():
+    """One rank's share of Ulysses SP=4 attention at its real shape: 65,536 tokens, 4 of the 16 heads, head_dim 80.
+    Windowed layout (64-token windows): everything against the oracle.  Full layer: the oracle's O(L^2) pass is
+    out of reach on the host, so sampled query rows (O, lse, dQ) and sampled key rows (dK, dV) are recomputed in
+    fp32 from their definitions; the key-row check takes lse and O for the non-sampled rows from the kernel."""
+    ops = _ops()
+    L, H, d = 65536, 4, 80
+    scale = d**-0.5
+    _announce("attention bf16 SP share, windows")
+    _attn_case(torch.bfloat16, [64] * 1024, H, d, seed=11)
+    _announce("attention bf16 SP share, full layer")
+    g = torch.Generator().manual_seed(12)
+    q, k, v, do = (torch.randn(L, H * d, generator=g).to(torch.bfloat16).to(DEV) for _ in range(4))
+    cu = torch.tensor([0, L], dtype=torch.int32, device=DEV)
+    o, lse = ops.attn_fwd(q, k, v, cu, L, H, d, scale)
+    dq, dk, dv = (torch.empty_like(q) for _ in range(3))
+    ops.attn_bwd(q, k, v, o, do, lse, cu, L, H, d, scale, dq, dk, dv)
+    idx = torch.randint(0, L, (48,), generator=g).to(DEV)
+    qf, kf, vf, dof, of = (t.float().reshape(L, H, d) for t in (q, k, v, do, o))
+    # sampled queries
+    s = torch.einsum("qhd,khd->hqk", qf[idx], kf) * scale
+    lse_ref = torch.logsumexp(s, dim=-1)  # [H, 48]
+    p = torch.exp(s - lse_ref[..., None])
+    o_ref = torch.einsum("hqk,khd->qhd", p, vf)
+    assert max_rel_err(o[idx].float().reshape(-1, H, d), o_ref) < TOL[torch.bfloat16], "forward rows"
+    assert torch.allclose(lse[:, idx], lse_ref, rtol=2e-3, atol=2e-3), "lse rows"
+    dp = torch.einsum("qhd,khd->hqk", dof[idx], vf)
+    delta = (dof[idx] * o_ref).sum(-1).transpose(0, 1)  # [H, 48]
+    ds = p * (dp - delta[..., None])
+    dq_ref = torch.einsum("hqk,khd->qhd", ds, kf) * scale
+    assert max_rel_err(dq[idx].float().reshape(-1, H, d), dq_ref) < TOL[torch.bfloat16], "dq rows"
+    # sampled keys
+    st = torch.einsum("qhd,khd->hqk", qf, kf[idx]) * scale  # [H, L, 48]
+    pt = torch.exp(st - lse[..., None])
+    dv_ref = torch.einsum("hqk,qhd->khd", pt, dof)
+    dpt = torch.einsum("qhd,khd->hqk", dof, vf[idx])
+    delta_all = (dof * of).sum(-1).transpose(0, 1)  # [H, L]
+    dk_ref = torch.einsum("hqk,qhd->khd", pt * (dpt - delta_all[..., None]), qf) * scale
+    assert max_rel_err(dv[idx].float().reshape(-1, H, d), dv_ref) < TOL[torch.bfloat16], "dv rows"
+    assert max_rel_err(dk[idx].float().reshape(-1, H, d), dk_ref) < TOL[torch.bfloat16], "dk rows"
 
 
 def test_attention_softmax_invariants():
