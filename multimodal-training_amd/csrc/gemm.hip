@@ -92,7 +92,8 @@ __device__ __forceinline__ float gelu_erf_grad(float z) {
   const float pdf = 0.39894228040143267794f * __expf(-0.5f * z * z);
   return cdf + z * pdf;
 }
-__device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + __expf(-z)); }
+// 1 / (1 + e^-z) with the hardware reciprocal (1 ulp) instead of the IEEE division sequence
+__device__ __forceinline__ float sigmoidf_(float z) { return __builtin_amdgcn_rcpf(1.f + __expf(-z)); }
 
 // 8 consecutive elements <-> fp32 registers
 __device__ __forceinline__ void load8(const bf16_t* p, float* v) {
