@@ -436,21 +436,27 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
   float* ws = to_ws ? p.workspace + (int64_t)slice * p.M * p.N : nullptr;
   const bool ws_vec = (p.N % 4 == 0);
 
-  // Tiles inside the matrix whose epilogue reads one value per output element: those reads run up to two passes
-  // ahead, so their latency hides behind the LDS staging and the previous passes' arithmetic and stores.
+  // Tiles inside the matrix: compile-time trip counts, no edge tests, 16-byte accesses only.  When the epilogue
+  // reads one value per output element, those reads run up to two passes ahead, so their latency hides behind
+  // the LDS staging and the previous passes' arithmetic and stores.
   using EP = EpiPre<T, EPI, BM, BN, WM, NTHREADS>;
-  if constexpr (EP::HAS_IN) {
-    if (ep.active) {
-      constexpr int ITEMS = EP::ITEMS;
+  if constexpr ((PASS_ROWS * GROUPS) % NTHREADS == 0) {
+    const bool interior = m0 + BM <= p.M && n0 + NCOLS <= p.N && (to_ws ? ws_vec : p.vec_ok != 0) && (!EP::HAS_IN || ep.active);
+    if (interior) {
+      constexpr int ITEMS = PASS_ROWS * GROUPS / NTHREADS;
       constexpr int NBUF = EP::NBUF;
-      ep.template fetch<0>(p, 0);
-      if (NBUF == 2 && MT > 1) ep.template fetch<(NBUF - 1)>(p, 1);
+      if constexpr (EP::HAS_IN) {
+        ep.template fetch<0>(p, 0);
+        if (NBUF == 2 && MT > 1) ep.template fetch<(NBUF - 1)>(p, 1);
+      }
 #pragma unroll
       for (int a = 0; a < MT; ++a) {
         if (a > 0) __syncthreads();
 #pragma unroll
         for (int b = 0; b < NT; ++b) {
-          const int col = wn * WN + b * 32 + lc;
+          int col;
+          if (DUAL) col = (b / (NT / 2)) * (BN / 2) + wn * (WN / 2) + (b % (NT / 2)) * 32 + lc;
+          else col = wn * WN + b * 32 + lc;
 #pragma unroll
           for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -460,14 +466,28 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
 #pragma unroll
         for (int it = 0; it < ITEMS; ++it) {
           const int c = threadIdx.x + NTHREADS * it, row = c / GROUPS, cg = c % GROUPS;
+          const int64_t m = m0 + (row / 32) * WM + a * 32 + (row % 32), n = n0 + cg * 8;
           const float* sp = stage + row * SP + cg * 8;
           const f32x4 v0 = *reinterpret_cast<const f32x4*>(sp), v1 = *reinterpret_cast<const f32x4*>(sp + 4);
           float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-          emit8_impl<T, TO, EPI, true, true>(p, m0 + (row / 32) * WM + a * 32 + (row % 32), n0 + cg * 8, v, nullptr, ep.pre[a % NBUF][it]);
+          float u[8];
+          if (DUAL) {
+            const f32x4 u0 = *reinterpret_cast<const f32x4*>(sp + BN / 2), u1 = *reinterpret_cast<const f32x4*>(sp + BN / 2 + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              u[e] = u0[e];
+              u[4 + e] = u1[e];
+            }
+          }
+          if (to_ws) store8(ws + m * p.N + n, v);
+          else if constexpr (EP::HAS_IN) emit8_impl<T, TO, EPI, true, true>(p, m, n, v, u, ep.pre[a % NBUF][it]);
+          else emit8_impl<T, TO, EPI, true, false>(p, m, n, v, u);
         }
-        if (a + NBUF < MT) {
-          if ((a % NBUF) == 1) ep.template fetch<(NBUF - 1)>(p, a + NBUF);
-          else ep.template fetch<0>(p, a + NBUF);
+        if constexpr (EP::HAS_IN) {
+          if (a + NBUF < MT) {
+            if ((a % NBUF) == 1) ep.template fetch<(NBUF - 1)>(p, a + NBUF);
+            else ep.template fetch<0>(p, a + NBUF);
+          }
         }
       }
       return;
