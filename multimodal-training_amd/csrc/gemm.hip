@@ -5,7 +5,6 @@
 //      filled by direct global -> LDS loads (see gemm_dl_kernel).
 //   1: 256x256 tile, 8 waves, BK = 64 (fp32: 16), global -> registers -> LDS, double-buffered LDS, one barrier
 //      per K step.  The fp32 parity path (v_mfma_f32_32x32x2_f32) and the fallback for huge leading dimensions.
-//   2: 256x128 tile, 4 waves, single LDS buffer, two work-groups per CU.
 // Operands whose contraction index is contiguous in memory are staged as [row][k] and read with 16-byte LDS
 // loads; operands whose contraction index is the slow dimension (dgrad's weight, both operands of wgrad) are
 // staged as [k][row] exactly as they lie in memory and read with ds_read_b64_tr_b16, which hands each lane 4
@@ -79,11 +78,7 @@ template <int VAR>
 struct Waves;
 template <>
 struct Waves<1> {  // 256x256 tile, 8 waves of 128x64, double-buffered LDS, one work-group per CU
-  static constexpr int BM = 256, BN = 256, WM = 128, WN = 64, NTHREADS = 512, STAGES = 2, MIN_WAVES = 2;
-};
-template <>
-struct Waves<2> {  // 256x128 tile, 4 waves of 128x64, single LDS buffer: two independent work-groups per CU
-  static constexpr int BM = 256, BN = 128, WM = 128, WN = 64, NTHREADS = 256, STAGES = 1, MIN_WAVES = 2;
+  static constexpr int BM = 256, BN = 256, WM = 128, WN = 64, NTHREADS = 512, MIN_WAVES = 2;
 };
 
 __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.f + erff(z * 0.70710678118654752440f)); }
@@ -544,7 +539,7 @@ template <typename T, typename TO, bool TA, bool TB, int EPI, int VAR>
 __global__ __launch_bounds__(Waves<VAR>::NTHREADS, Waves<VAR>::MIN_WAVES) void gemm_kernel(const GemmParams p) {
   using C = Cfg<T>;
   using W = Waves<VAR>;
-  constexpr int BK = C::BK, BM = W::BM, BN = W::BN, WM = W::WM, WN = W::WN, NTHREADS = W::NTHREADS, STAGES = W::STAGES;
+  constexpr int BK = C::BK, BM = W::BM, BN = W::BN, WM = W::WM, WN = W::WN, NTHREADS = W::NTHREADS;
   constexpr int MT = WM / 32, NT = WN / 32, WGN = BN / WN;  // waves along N
   constexpr bool DUAL = (EPI == MVIT_EPI_SWIGLU);
   using LoaderA = TileLoader<T, BM, TA, NTHREADS, WN, false>;
@@ -589,21 +584,13 @@ __global__ __launch_bounds__(Waves<VAR>::NTHREADS, Waves<VAR>::MIN_WAVES) void g
   lb.init(B, B2, p.ldb, n0, p.N, k_begin, k_end);
   la.load();
   lb.load();
-  if (STAGES == 2) {
-    la.store(lds);
-    lb.store(lds + LoaderA::LDS_ELEMS);
-    __syncthreads();
-  }
+  la.store(lds);
+  lb.store(lds + LoaderA::LDS_ELEMS);
+  __syncthreads();
 
   int buf = 0;
   for (int64_t k0 = k_begin; k0 < k_end; k0 += BK) {
     const bool has_next = k0 + BK < k_end;
-    if (STAGES == 1) {
-      if (k0 > k_begin) __syncthreads();  // the previous tile has been consumed by every wave
-      la.store(lds);
-      lb.store(lds + LoaderA::LDS_ELEMS);
-      __syncthreads();
-    }
     if (has_next) {
       la.load();
       lb.load();
@@ -650,17 +637,14 @@ __global__ __launch_bounds__(Waves<VAR>::NTHREADS, Waves<VAR>::MIN_WAVES) void g
           for (int b = 0; b < NT; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a], fb[b], acc[a][b], 0, 0, 0);
       }
     }
-    if (STAGES == 2) {
-      if (has_next) {
-        T* nxt = lds + (buf ^ 1) * STAGE_ELEMS;
-        la.store(nxt);
-        lb.store(nxt + LoaderA::LDS_ELEMS);
-      }
-      __syncthreads();
-      buf ^= 1;
+    if (has_next) {
+      T* nxt = lds + (buf ^ 1) * STAGE_ELEMS;
+      la.store(nxt);
+      lb.store(nxt + LoaderA::LDS_ELEMS);
     }
+    __syncthreads();  // also: operands fully consumed before LDS is reused by the epilogue
+    buf ^= 1;
   }
-  if (STAGES == 1) __syncthreads();  // operands fully consumed before LDS is reused for the epilogue
 
   EpiPre<T, EPI, BM, BN, WM, NTHREADS> ep;
   ep.init(p, m0, n0);
@@ -799,9 +783,7 @@ __device__ __forceinline__ void wait_tiles(int n) {
   else wait_vm<0>();
 }
 
-// PF: the first 16-wide step's operands of tile t+1 are fetched from LDS while tile t's second step runs on the
-// MFMAs; tile t+1 must then have landed one barrier earlier, so one tile less is in flight.
-template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, bool PF, int NW>
+template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, int NW>
 __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmParams p) {
   using T = bf16_t;
   using D = DL<NW>;
@@ -865,33 +847,23 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
   for (int t = 0; t < NSTAGE - 1; ++t) issue(t, t);
 
   bf16x8 fa[2][MT], fb[2][NT];
-  if (PF && T_ > 0) {
-    wait_tiles<2 * D::CPT>(T_ - 1 < NSTAGE - 2 ? T_ - 1 : NSTAGE - 2);
-    __builtin_amdgcn_s_barrier();
-#pragma unroll
-    for (int a = 0; a < MT; ++a) fa[0][a] = ra.read(smem_raw, a, 0, 0);
-#pragma unroll
-    for (int b = 0; b < NT; ++b) fb[0][b] = rb.read(smem_raw, b, 0, 0);
-  }
   for (int t0 = 0; t0 < T_; t0 += NSTAGE) {
 #pragma unroll
     for (int s = 0; s < NSTAGE; ++s) {
       const int t = t0 + s;
       if (t >= T_) break;
-      // tile t (PF: t+1) has landed once only the tiles issued after it are pending
-      const int rem = T_ - 1 - t - (PF ? 1 : 0);
-      constexpr int AHEAD = NSTAGE - 2 - (PF ? 1 : 0);
+      // tile t has landed once only the tiles issued after it are pending
+      const int rem = T_ - 1 - t;
+      constexpr int AHEAD = NSTAGE - 2;
       wait_tiles<2 * D::CPT>(rem < 0 ? 0 : (rem < AHEAD ? rem : AHEAD));
       __builtin_amdgcn_s_barrier();  // every wave's share of that tile is in LDS; stage (s-1) has been consumed
       issue(t + NSTAGE - 1, (s + NSTAGE - 1) % NSTAGE);
 
-      if (!PF) {
 #pragma unroll
-        for (int a = 0; a < MT; ++a) fa[0][a] = ra.read(smem_raw, a, 0, s);
+      for (int a = 0; a < MT; ++a) fa[0][a] = ra.read(smem_raw, a, 0, s);
 #pragma unroll
-        for (int b = 0; b < NT; ++b) fb[0][b] = rb.read(smem_raw, b, 0, s);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+      for (int b = 0; b < NT; ++b) fb[0][b] = rb.read(smem_raw, b, 0, s);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int a = 0; a < MT; ++a) fa[1][a] = ra.read(smem_raw, a, 1, s);
 #pragma unroll
@@ -903,13 +875,6 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
         for (int b = 0; b < NT; ++b)
           acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0][a], fb[0][b], acc[a][b], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
-      if (PF && t + 1 < T_) {
-#pragma unroll
-        for (int a = 0; a < MT; ++a) fa[0][a] = ra.read(smem_raw, a, 0, (s + 1) % NSTAGE);
-#pragma unroll
-        for (int b = 0; b < NT; ++b) fb[0][b] = rb.read(smem_raw, b, 0, (s + 1) % NSTAGE);
-        __builtin_amdgcn_sched_barrier(0);
-      }
 #pragma unroll
       for (int a = 0; a < MT; ++a)
 #pragma unroll
@@ -942,7 +907,7 @@ int launch(const GemmParams& p, hipStream_t stream) {
   constexpr int BM = W::BM, BN = W::BN;
   using LA = TileLoader<T, BM, TA, W::NTHREADS, W::WN, false>;
   using LB = TileLoader<T, BN, TB, W::NTHREADS, W::WN, false>;
-  const size_t operands = W::STAGES * (size_t)(LA::LDS_ELEMS + LB::LDS_ELEMS) * sizeof(T);
+  const size_t operands = 2 * (size_t)(LA::LDS_ELEMS + LB::LDS_ELEMS) * sizeof(T);
   const size_t staging = (size_t)(BM / W::WM) * 32 * (BN + 8) * sizeof(float);
   const size_t lds = operands > staging ? operands : staging;
   auto kern = gemm_kernel<T, TO, TA, TB, EPI, VAR>;
@@ -966,13 +931,13 @@ int launch(const GemmParams& p, hipStream_t stream) {
   return MVIT_OK;
 }
 
-template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, bool PF, int NW>
+template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, int NW>
 int launch_dl(const GemmParams& p, hipStream_t stream) {
   using D = DL<NW>;
   const size_t operands = 2 * (size_t)NSTAGE * D::TILE_BYTES;
   const size_t staging = (size_t)(D::BM / D::WM) * 32 * (D::BN + 8) * sizeof(float);
   const size_t lds = operands > staging ? operands : staging;
-  auto kern = gemm_dl_kernel<TO, TA, TB, EPI, NSTAGE, PF, NW>;
+  auto kern = gemm_dl_kernel<TO, TA, TB, EPI, NSTAGE, NW>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -1003,11 +968,10 @@ int launch_dl(const GemmParams& p, hipStream_t stream) {
 template <typename T, typename TO, bool TA, bool TB, int EPI>
 int launch_var(int var, const GemmParams& p, hipStream_t s) {
   if constexpr (sizeof(T) == 2) {
-    if (var == 3) return launch_dl<TO, TA, TB, EPI, 4, false, 8>(p, s);
+    if (var == 3) return launch_dl<TO, TA, TB, EPI, 4, 8>(p, s);
 
   }
   if (var == 1 || var >= 3) return launch<T, TO, TA, TB, EPI, 1>(p, s);
-  if (var == 2) return launch<T, TO, TA, TB, EPI, 2>(p, s);
   return launch<T, TO, TA, TB, EPI, 1>(p, s);
 }
 
@@ -1082,9 +1046,9 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
   const size_t es = a->dtype == MVIT_BF16 ? 2 : 4, eo = a->out_dtype == MVIT_BF16 ? 2 : 4;
   p.vec_ok = vec16(a->C, a->ldc, eo) && vec16(a->R, a->ldr, es) && vec16(a->aux, a->ldaux, es) && vec16(a->bias, 0, es) &&
              vec16(a->bias2, 0, es) && (a->aux_off * (int64_t)(es < eo ? es : eo)) % 16 == 0;
-  int var = (a->reserved >= 1 && a->reserved <= 3) ? a->reserved : 3;  // 0 = default
+  int var = (a->reserved == 1 || a->reserved == 3) ? a->reserved : 3;  // 0 (or anything else) = default
   if (var >= 3 && (a->lda > (1ll << 22) || a->ldb > (1ll << 22))) var = 1;  // 32-bit lane offsets  // tile / wave layout, see Waves<>
-  const int BM = 256, BN = var == 2 ? 128 : 256;
+  const int BM = 256, BN = 256;
   const int n_per_block = (epi == MVIT_EPI_SWIGLU) ? BN / 2 : BN;
   const int64_t tm = (a->M + BM - 1) / BM, tn = (a->N + n_per_block - 1) / n_per_block;
   MVIT_REQUIRE(tm * tn < (1ll << 30), "gemm: too many tiles");
