@@ -150,7 +150,9 @@ typedef struct mvit_gemm_args {
   void* aux;
   int64_t ldaux;
   int64_t aux_off; /* column offset of the second half in aux (SWIGLU) / R and C (SWIGLU_BWD) */
-  void* workspace; /* fp32 scratch of split_k * M * N floats when split_k > 1, else unused */
+  void* workspace; /* split_k > 1: fp32 scratch of split_k * M * N floats.  MVIT_EPI_SWIGLU_BWD (optional): receives
+                      fp32 column sums of C per 256-row tile, [ceil(M/256)][ldc] (columns [0,N) and
+                      [aux_off, aux_off+N) are written); add the rows with mvit_reduce_partials for the bias gradient */
   int64_t workspace_bytes;
   int split_k;   /* <= 1: one work-group per tile walks all of K.  > 1 (EPI_NONE only): K is cut in split_k slices
                     whose fp32 partial tiles go to `workspace` and are summed by a second kernel (fixed order) */

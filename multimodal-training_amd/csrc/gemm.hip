@@ -38,6 +38,7 @@ struct GemmParams {
   int64_t k_chunk;    // K extent of one slice (multiple of BK)
   float* workspace;   // [split_k][M][N] fp32 partial sums when split_k > 1
   int vec_ok;         // every epilogue pointer / stride allows 16-byte accesses
+  float* colsum;      // SWIGLU_BWD: per-tile-row column sums of the output, [tiles_m][ldc] (null: not wanted)
   int flags;          // tuning switches: 2 = one work-group per tile instead of persistent work-groups
   int panel_w;        // tiles are walked in panels of this many tile columns (M fastest across a panel's rows)
 };
@@ -250,7 +251,7 @@ __device__ __forceinline__ float frag_f32(const float* lds, int row, int k) {
 // PRE: the epilogue's per-element inputs (residual / saved activations) were fetched earlier into pre[0..1].
 template <typename T, typename TO, int EPI, bool FULL, bool PRE = false>
 __device__ __forceinline__ void emit8_impl(const GemmParams& p, int64_t m, int64_t n, float* v, const float* u,
-                                           const T __attribute__((ext_vector_type(8))) * pre = nullptr) {
+                                           const T __attribute__((ext_vector_type(8))) * pre, float (&cs)[16], bool do_cs) {
   TO* Cp = static_cast<TO*>(p.C);
   const T* Rp = static_cast<const T*>(p.R);
   T* auxp = static_cast<T*>(p.aux);
@@ -322,6 +323,15 @@ __device__ __forceinline__ void emit8_impl(const GemmParams& p, int64_t m, int64
       dg[e] = v[e] * uu[e] * (sg + silu * (1.f - sg));
       du[e] = v[e] * silu;
     }
+    if (do_cs) {  // running column sums of this thread's 8 columns (the gate / up bias gradient)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (e < cnt) {
+          cs[e] += dg[e];
+          cs[8 + e] += du[e];
+        }
+      }
+    }
     TO* dg_out = Cp + m * p.ldc + n;
     TO* du_out = dg_out + p.aux_off;
     if (vec) {
@@ -368,9 +378,10 @@ __device__ __forceinline__ void emit8_impl(const GemmParams& p, int64_t m, int64
 }
 
 template <typename T, typename TO, int EPI>
-__device__ __forceinline__ void emit8(const GemmParams& p, int64_t m, int64_t n, float* v, const float* u, bool vec) {
-  if (vec && n + 8 <= p.N) emit8_impl<T, TO, EPI, true>(p, m, n, v, u);
-  else emit8_impl<T, TO, EPI, false>(p, m, n, v, u);
+__device__ __forceinline__ void emit8(const GemmParams& p, int64_t m, int64_t n, float* v, const float* u, bool vec,
+                                      float (&cs)[16], bool do_cs) {
+  if (vec && n + 8 <= p.N) emit8_impl<T, TO, EPI, true>(p, m, n, v, u, nullptr, cs, do_cs);
+  else emit8_impl<T, TO, EPI, false>(p, m, n, v, u, nullptr, cs, do_cs);
 }
 
 // Per-element epilogue inputs (residual / saved activations) of an interior tile, fetched ahead of their use.
@@ -430,6 +441,33 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
   const bool to_ws = (EPI == MVIT_EPI_NONE) && p.split_k > 1;
   float* ws = to_ws ? p.workspace + (int64_t)slice * p.M * p.N : nullptr;
   const bool ws_vec = (p.N % 4 == 0);
+  // SWIGLU_BWD can hand back the column sums of dg | du (the bias gradient): a thread's items all lie in the same
+  // 8 columns, so it keeps 2 x 8 running sums; after the last pass the rows-of-threads are added through LDS.
+  constexpr bool CAN_CS = (EPI == MVIT_EPI_SWIGLU_BWD) && NTHREADS % GROUPS == 0 && NTHREADS == 2 * GROUPS * 8;
+  float cs_acc[16];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) cs_acc[e] = 0.f;
+  const bool do_cs = CAN_CS && p.colsum != nullptr;
+  auto finish_colsum = [&]() {
+    if constexpr (CAN_CS) {
+      if (!do_cs) return;
+      constexpr int TR_ = NTHREADS / GROUPS;  // thread rows sharing a column group
+      __syncthreads();                        // the staging area is free
+      float* red = stage;                     // [TR_][2][GROUPS * 8]
+      const int trow = threadIdx.x / GROUPS, cgx = threadIdx.x % GROUPS;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        red[(trow * 2 + 0) * (GROUPS * 8) + cgx * 8 + e] = cs_acc[e];
+        red[(trow * 2 + 1) * (GROUPS * 8) + cgx * 8 + e] = cs_acc[8 + e];
+      }
+      __syncthreads();
+      const int half = threadIdx.x / (GROUPS * 8), col = threadIdx.x % (GROUPS * 8);  // NTHREADS == 2 * GROUPS * 8
+      float t = 0.f;
+#pragma unroll
+      for (int k = 0; k < TR_; ++k) t += red[(k * 2 + half) * (GROUPS * 8) + col];
+      if (n0 + col < p.N) p.colsum[(m0 / BM) * p.ldc + (half ? p.aux_off : 0) + n0 + col] = t;
+    }
+  };
 
   // Tiles inside the matrix: compile-time trip counts, no edge tests, 16-byte accesses only.  When the epilogue
   // reads one value per output element, those reads run up to two passes ahead, so their latency hides behind
@@ -475,8 +513,8 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
             }
           }
           if (to_ws) store8(ws + m * p.N + n, v);
-          else if constexpr (EP::HAS_IN) emit8_impl<T, TO, EPI, true, true>(p, m, n, v, u, ep.pre[a % NBUF][it]);
-          else emit8_impl<T, TO, EPI, true, false>(p, m, n, v, u);
+          else if constexpr (EP::HAS_IN) emit8_impl<T, TO, EPI, true, true>(p, m, n, v, u, ep.pre[a % NBUF][it], cs_acc, do_cs);
+          else emit8_impl<T, TO, EPI, true, false>(p, m, n, v, u, nullptr, cs_acc, false);
         }
         if constexpr (EP::HAS_IN) {
           if (a + NBUF < MT) {
@@ -485,6 +523,7 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
           }
         }
       }
+      finish_colsum();
       return;
     }
   }
@@ -529,10 +568,11 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
         else
           for (int e = 0; e < 8 && n + e < p.N; ++e) w[e] = v[e];
       } else {
-        emit8<T, TO, EPI>(p, m, n, v, u, p.vec_ok != 0);
+        emit8<T, TO, EPI>(p, m, n, v, u, p.vec_ok != 0, cs_acc, do_cs);
       }
     }
   }
+  finish_colsum();
 }
 
 template <typename T, typename TO, bool TA, bool TB, int EPI, int VAR>
@@ -1057,6 +1097,12 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
   p.flags = (a->reserved2 >> 8) & 0xff;
   if ((a->reserved2 & 0xff) > 0) p.panel_w = (a->reserved2 & 0xff) < tn ? (a->reserved2 & 0xff) : (int)tn;  // tuning override
   p.split_k = 1; p.k_chunk = a->K; p.workspace = nullptr;
+  p.colsum = nullptr;
+  if (epi == MVIT_EPI_SWIGLU_BWD && a->workspace) {
+    MVIT_REQUIRE(mvit_aligned16(a->workspace) && a->workspace_bytes >= (int64_t)sizeof(float) * tm * a->ldc,
+                 "gemm: SWIGLU_BWD column sums need a workspace of %lld bytes", (long long)(sizeof(float) * tm * a->ldc));
+    p.colsum = static_cast<float*>(a->workspace);
+  }
   if (a->split_k > 1) {
     const int bk = a->dtype == MVIT_BF16 ? 64 : 16;
     const int64_t chunk = ((a->K + a->split_k - 1) / a->split_k + bk - 1) / bk * bk;

@@ -133,8 +133,10 @@ def _block_backward(dx2: torch.Tensor, x: torch.Tensor, saved: tuple, W: BlockWe
     g_wd = torch.empty(C, I, dtype=gdt["mlp.down_proj.weight"], device=dev)
     ops.gemm(dx2, h, g_wd, trans_a=True, trans_b=True, n=I, split_k=ops.wgrad_split_k(C, I, S))
     dgu = torch.empty(S, 2 * Ipad, dtype=x.dtype, device=dev)
-    ops.gemm(dx2, W.wdown, dgu, trans_b=True, epilogue=E.EPI_SWIGLU_BWD, residual=gu, aux_off=Ipad)
-    g_bgu = ops.colsum(dgu, gdt["mlp.gate_proj.bias"])
+    # the epilogue also hands back per-tile column sums of dgu: the gate / up bias gradient without re-reading dgu
+    part = torch.empty(-(-S // 256), 2 * Ipad, dtype=torch.float32, device=dev)
+    ops.gemm(dx2, W.wdown, dgu, trans_b=True, epilogue=E.EPI_SWIGLU_BWD, residual=gu, aux_off=Ipad, colsum_partial=part)
+    g_bgu = ops.reduce_partials(part, gdt["mlp.gate_proj.bias"])
     g_wgu = torch.empty(2 * Ipad, C, dtype=gdt["mlp.gate_proj.weight"], device=dev)
     ops.gemm(dgu, n2, g_wgu, trans_a=True, trans_b=True, split_k=ops.wgrad_split_k(2 * Ipad, C, S))
     dn2 = torch.empty_like(x)

@@ -144,6 +144,16 @@ def rmsnorm_bwd(dy, x, w, rstd, dx_add: Optional[torch.Tensor] = None, w_grad_dt
     return dx, dw
 
 
+def reduce_partials(partial: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """Column sums of a contiguous fp32 [n_partial, cols] array of partial sums (fixed order, reproducible)."""
+    if partial.dtype != torch.float32 or partial.dim() != 2 or not partial.is_contiguous():
+        raise ValueError("reduce_partials: expected a contiguous fp32 2-D tensor")
+    out = torch.empty(partial.shape[1], dtype=out_dtype, device=partial.device)
+    rc = _lib.load().mvit_reduce_partials(partial.data_ptr(), partial.shape[0], partial.shape[1], out.data_ptr(), dt(out), _stream(partial))
+    _lib.check(rc, "mvit_reduce_partials")
+    return out
+
+
 def colsum(x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
     """Column sums of a 2-D (possibly row-strided) tensor: the bias gradient of a Linear layer."""
     _rowmajor(x, "colsum x")
@@ -259,11 +269,13 @@ def gemm(
     aux_off: int = 0,
     n: Optional[int] = None,
     split_k: int = 1,
+    colsum_partial: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """out[M, N] = epilogue(A . B^T) with A = a (or a^T if trans_a) and B = b (or b^T if trans_b), see include/mi355_vit.h.
 
     Shapes: a [M,K] (or [K,M]); b [N,K] (or [K,N]); all 2-D with unit column stride (row strides free).
     ``n`` narrows the logical N (columns of B / out) below b's extent.
+    ``colsum_partial`` (EPI_SWIGLU_BWD only): fp32 [ceil(M/256), out.stride(0)] receiving per-tile column sums of out.
     """
     for t, nm in ((a, "a"), (b, "b"), (out, "out")):
         _rowmajor(t, f"gemm {nm}")
@@ -312,6 +324,13 @@ def gemm(
             raise ValueError("gemm: split_k needs the plain epilogue")
         ws = torch.empty(split_k * M * N, dtype=torch.float32, device=a.device)
         args.workspace, args.workspace_bytes, args.split_k = ws.data_ptr(), ws.numel() * 4, split_k
+    if colsum_partial is not None:
+        if epilogue != _lib.EPI_SWIGLU_BWD:
+            raise ValueError("gemm: colsum_partial is an output of the SwiGLU-backward epilogue only")
+        cp = colsum_partial
+        if cp.dtype != torch.float32 or not cp.is_contiguous() or cp.shape != (-(-M // 256), out.stride(0)) or cp.device != a.device:
+            raise ValueError(f"gemm: colsum_partial must be contiguous fp32 [{-(-M // 256)}, {out.stride(0)}]")
+        args.workspace, args.workspace_bytes = cp.data_ptr(), cp.numel() * 4
     st = _stream(a)
     tag = f"gemm_{'t' if trans_a else 'n'}{'t' if trans_b else 'n'}_epi{epilogue}"
     _lib.check(_launch(tag, {"M": M, "N": N, "K": K}, lambda: _lib.load().mvit_gemm(C.byref(args), st)), "mvit_gemm")

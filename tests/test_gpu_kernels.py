@@ -322,7 +322,11 @@ def test_gemm_gelu_and_swiglu_epilogues(dtype):
     dx, wd = _rand((M, Cc), dtype, 9), torch.zeros(Cc, Ipad, dtype=dtype)
     wd[:, :I] = _rand((Cc, I), dtype, 10, I**-0.5)
     dgu = torch.full((M, 2 * Ipad), float("nan"), dtype=dtype, device=DEV)
-    ops.gemm(dx.to(DEV), wd.to(DEV), dgu, trans_b=True, epilogue=E.EPI_SWIGLU_BWD, residual=gu, aux_off=Ipad)
+    part = torch.full((-(-M // 256), 2 * Ipad), float("nan"), dtype=torch.float32, device=DEV)
+    ops.gemm(dx.to(DEV), wd.to(DEV), dgu, trans_b=True, epilogue=E.EPI_SWIGLU_BWD, residual=gu, aux_off=Ipad, colsum_partial=part)
+    # fused bias gradient: column sums of dgu, accumulated in fp32 before the rounding to the storage type
+    bsum = ops.reduce_partials(part, torch.float32)
+    assert max_rel_err(bsum, dgu.float().sum(0)) < TOL[dtype]
     g0 = gu[:, :I].float().cpu().requires_grad_(True)
     u0 = gu[:, Ipad : Ipad + I].float().cpu().requires_grad_(True)
     (F.silu(g0) * u0).backward(dx.float() @ wd.float()[:, :I])
