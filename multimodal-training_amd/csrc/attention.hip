@@ -842,10 +842,10 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams
 // (segment, head) are staged in LDS once.  Pass A works in the dQ orientation (a lane owns a query), where
 // delta_q = sum_k P[q,k] * dP[q,k] (equal to dO_q . O_q, so O is never read) is a lane-local sum, and writes dQ;
 // pass B repeats the dK/dV kernel's tile loop on the staged tiles.  HBM traffic: four tiles in, three out.
-template <int ND>
-__global__ __launch_bounds__(64) void attn_bwd_window_mfma(const AttnParams p) {
+template <int ND, int NW>  // NW waves share the staged tiles; wave w owns query / key blocks [w*4/NW, (w+1)*4/NW)
+__global__ __launch_bounds__(64 * NW) void attn_bwd_window_mfma(const AttnParams p) {
   using G = Geo<ND>;
-  constexpr int HD = G::HD, R = 64, PK = G::PK;
+  constexpr int HD = G::HD, R = 64, PK = G::PK, NB = 4 / NW;  // NB 16-row blocks per wave
   __shared__ __attribute__((aligned(16))) bf16_t lds_q[R * PK];
   __shared__ __attribute__((aligned(16))) bf16_t lds_k[R * PK];
   __shared__ __attribute__((aligned(16))) bf16_t lds_v[R * PK];
@@ -857,10 +857,10 @@ __global__ __launch_bounds__(64) void attn_bwd_window_mfma(const AttnParams p) {
   const int s0 = p.cu[seg];
   const int L = min(p.cu[seg + 1] - s0, R);
   if (L <= 0) return;
-  const int l = threadIdx.x, g = l >> 4, r = l & 15;
+  const int l = threadIdx.x & 63, wv = threadIdx.x >> 6, g = l >> 4, r = l & 15;
   const float c = p.scale * LOG2E;
   {
-    TileStager<ND, R, PK, 64> sq, sk, sv, sdo;
+    TileStager<ND, R, PK, 64 * NW> sq, sk, sv, sdo;
     sq.init(p.q_stride);
     sk.init(p.k_stride);
     sv.init(p.v_stride);
@@ -869,7 +869,7 @@ __global__ __launch_bounds__(64) void attn_bwd_window_mfma(const AttnParams p) {
     sk.load(static_cast<const bf16_t*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD, L);
     sv.load(static_cast<const bf16_t*>(p.v) + (int64_t)s0 * p.v_stride + (int64_t)h * HD, L);
     sdo.load(static_cast<const bf16_t*>(p.d_o) + (int64_t)s0 * p.do_stride + (int64_t)h * HD, L);
-    lds_lse[l] = l < L ? p.lse[(int64_t)h * p.total + s0 + l] * LOG2E : INFINITY;  // +inf => p = 0 for padded queries
+    if (wv == 0) lds_lse[l] = l < L ? p.lse[(int64_t)h * p.total + s0 + l] * LOG2E : INFINITY;  // +inf => p = 0 for padded queries
     sq.scale(c);  // the Q tile holds Q * scale * log2(e): scores leave the MFMA in log2 units
     sq.store(lds_q);
     sk.store(lds_k);
@@ -898,7 +898,7 @@ __global__ __launch_bounds__(64) void attn_bwd_window_mfma(const AttnParams p) {
     bf16_t* DQ = static_cast<bf16_t*>(p.dq) + (int64_t)s0 * p.dq_stride + (int64_t)h * HD;
     float* DELTA = p.delta + (int64_t)h * p.total + s0;
 #pragma unroll 1
-    for (int qb = 0; qb < 4; ++qb) {
+    for (int qb = wv * NB; qb < (wv + 1) * NB; ++qb) {
       if (qb * 16 >= L) break;
       const int qi = qb * 16 + r;
       RowFrag<ND> qf, dof;
@@ -951,18 +951,19 @@ __global__ __launch_bounds__(64) void attn_bwd_window_mfma(const AttnParams p) {
         }
       }
     }
-    for (int q = 16 * ((L + 15) / 16) + l; q < R; q += 64) lds_delta[q] = 0.f;  // query blocks that were skipped
+    for (int q = 16 * ((L + 15) / 16) + (int)threadIdx.x; q < R; q += 64 * NW) lds_delta[q] = 0.f;  // query blocks that were skipped
   }
   __syncthreads();
 
   // ---- pass B: dV^T += dO^T P, dK^T += Q^T dS per 16-key block, queries in two tiles of 32
   {
-    RowFrag<ND> kf[4], vf[4];
-    f32x4 dk[4][ND], dv[4][ND];
+    RowFrag<ND> kf[NB], vf[NB];
+    f32x4 dk[NB][ND], dv[NB][ND];
+    const int key0 = wv * NB * 16;  // this wave's first key
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
-      load_rowfrag_lds<ND, PK>(kf[kb], lds_k, kb * 16 + r, g);
-      load_rowfrag_lds<ND, PK>(vf[kb], lds_v, kb * 16 + r, g);
+    for (int kb = 0; kb < NB; ++kb) {
+      load_rowfrag_lds<ND, PK>(kf[kb], lds_k, key0 + kb * 16 + r, g);
+      load_rowfrag_lds<ND, PK>(vf[kb], lds_v, key0 + kb * 16 + r, g);
 #pragma unroll
       for (int d = 0; d < ND; ++d) {
         dk[kb][d] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -990,7 +991,7 @@ __global__ __launch_bounds__(64) void attn_bwd_window_mfma(const AttnParams p) {
         dt_[d] = tr_pair(tdo + off, tdo + off + 16 * PK);
       }
 #pragma unroll
-      for (int kb = 0; kb < 4; ++kb) {
+      for (int kb = 0; kb < NB; ++kb) {
         f32x4 pv[2], ds[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -1015,8 +1016,8 @@ __global__ __launch_bounds__(64) void attn_bwd_window_mfma(const AttnParams p) {
     bf16_t* DK = static_cast<bf16_t*>(p.dk) + (int64_t)s0 * p.dk_stride + (int64_t)h * HD;
     bf16_t* DV = static_cast<bf16_t*>(p.dv) + (int64_t)s0 * p.dv_stride + (int64_t)h * HD;
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
-      const int ki = kb * 16 + r;
+    for (int kb = 0; kb < NB; ++kb) {
+      const int ki = key0 + kb * 16 + r;
       if (ki < L) {
 #pragma unroll
         for (int d = 0; d < ND; ++d) {
@@ -1223,7 +1224,10 @@ template <int ND>
 int launch_fwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t s) {
   const int nw = pick_waves(max_seqlen);
   dim3 grid((unsigned)((max_seqlen + 64 * nw - 1) / (64 * nw)), (unsigned)n_seg, (unsigned)p.nheads);
-  if (nw == 1) hipLaunchKernelGGL((attn_fwd_mfma<ND, 1, 64, false>), grid, 64, 0, s, p);
+  if (nw == 1 && ND <= 5) {
+    // windows: two waves x 32 queries share the staged K / V tiles (more waves per CU hide the load latency)
+    if constexpr (ND <= 5) hipLaunchKernelGGL((attn_fwd_mfma<ND, 2, 64, false, 2, 4>), grid, 128, 0, s, p);
+  } else if (nw == 1) hipLaunchKernelGGL((attn_fwd_mfma<ND, 1, 64, false>), grid, 64, 0, s, p);
   else if (nw == 2) hipLaunchKernelGGL((attn_fwd_mfma<ND, 2, 64, false>), grid, 128, 0, s, p);
   else if constexpr (ND <= 5) {
     // long segments: 8 waves x 32 queries, <= 128 registers, so that four waves share a SIMD and cover each
@@ -1240,7 +1244,7 @@ int launch_bwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
   if (max_seqlen <= 64) {
     dim3 grid(1, (unsigned)n_seg, (unsigned)p.nheads);
     if constexpr (ND <= 5) {
-      hipLaunchKernelGGL((attn_bwd_window_mfma<ND>), grid, 64, 0, s, p);  // computes delta itself
+      hipLaunchKernelGGL((attn_bwd_window_mfma<ND, 2>), grid, 128, 0, s, p);  // computes delta itself
     } else {
       hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 1, 4>), grid, 64, 0, s, p);
       hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 1, 4>), grid, 64, 0, s, p);
