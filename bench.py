@@ -93,8 +93,8 @@ def summarise_trace(records, cfg_kw, dtype):
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, scaled by what the same
 # counters read for a 1 GiB device copy: x2.000 and x1.000), keyed by (workload, trace tag).  The weight-gradient
-# launch is the GEMM kernel (544.1 MB) plus its split-K reduction (98.4 MB).
-MEASURED_TRAFFIC_BYTES = {("cfg2", "gemm_tt_epi0"): 642.5e6}
+# launch is the GEMM kernel (544.2 MB) plus its split-K reduction (98.4 MB).
+MEASURED_TRAFFIC_BYTES = {("cfg2", "gemm_tt_epi0"): 642.6e6}
 
 KERNEL_NAMES = {
     "gemm_nn_epi0": "gemm_dl_kernel<TO, TA=false, TB=false, EPI=NONE>",
@@ -106,10 +106,10 @@ KERNEL_NAMES = {
     "gemm_nt_epi5": "gemm_dl_kernel<TO, TA=false, TB=true, EPI=SWIGLU_BWD>",
     "gemm_nt_epi6": "gemm_dl_kernel<TO, TA=false, TB=true, EPI=GELU_BWD>",
     "gemm_tt_epi0": "gemm_dl_kernel<TO, TA=true, TB=true, EPI=NONE> + splitk_reduce_kernel",
-    "attn_fwd_full": "attn_fwd_mfma<5, 4, 32, true>",
+    "attn_fwd_full": "attn_fwd_mfma<5, 8, 32, true, 2, 4>",
     "attn_bwd_full": "attn_delta_kernel + attn_bwd_dkdv_mfma<5, 8, 2> + attn_bwd_dq_mfma<5, 8, 2>",
-    "attn_fwd_window": "attn_fwd_mfma<5, 1, 64, false>",
-    "attn_bwd_window": "attn_delta_kernel + attn_bwd_dkdv_mfma<5, 1, 4> + attn_bwd_dq_mfma<5, 1, 4>",
+    "attn_fwd_window": "attn_fwd_mfma<5, 2, 64, false, 2, 4>",
+    "attn_bwd_window": "attn_bwd_window_mfma<5, 2>",
 }
 
 
