@@ -167,6 +167,9 @@ def main() -> None:
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-trace", action="store_true", help="skip the per-kernel event pass (for profiler runs)")
+    ap.add_argument("--single-stream", action="store_true",
+                    help="run weight / bias gradients in line on the main stream instead of on the second stream (for profiler "
+                         "runs: kernels then never share the GPU, so their traced durations are their own)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain device copy of 1 GiB (8 launches) so that profiler byte counters can be scaled to a known size")
     args = ap.parse_args()
@@ -187,6 +190,8 @@ def main() -> None:
     from mi355_vit.config import Qwen2_5_VLVisionConfig
     from mi355_vit.modeling import Qwen2_5_VisionTransformerPretrainedModel
 
+    if args.single_stream:
+        ops.OVERLAP_WGRAD = False
     desc, cfg_kw, dtype, grid, seed, ckpt = make_workload(args.workload)
     dev = torch.device("cuda:0")
     torch.manual_seed(seed)
@@ -262,7 +267,8 @@ def main() -> None:
         "dtype": "bf16" if dtype == torch.bfloat16 else "f32",
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: {desc}", "patches": S, "grid_thw": grid.tolist(),
-                   "activation_checkpointing": ckpt, "peak_mem_gb": round(peak_mem_gb, 2)},
+                   "activation_checkpointing": ckpt, "peak_mem_gb": round(peak_mem_gb, 2),
+                   "streams": 2 if ops.OVERLAP_WGRAD else 1},
         "attention_mfma_util": attn_util,
         "roofline": roofline,
         "cpu_baseline": cpu,

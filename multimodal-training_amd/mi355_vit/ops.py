@@ -28,6 +28,22 @@ def set_trace(records: Optional[list]) -> None:
     _trace = records
 
 
+_side_streams: dict = {}
+OVERLAP_WGRAD = _os.environ.get("MVIT_OVERLAP", "1") != "0"
+
+
+def side_stream(device: torch.device) -> Optional["torch.cuda.Stream"]:
+    """The second stream (default priority) that weight-gradient GEMMs run on so that they fill the idle compute
+    units of the input-gradient chain; None while launches are being timed one by one."""
+    if not OVERLAP_WGRAD or _trace is not None:
+        return None
+    key = torch.device(device).index if torch.device(device).index is not None else torch.cuda.current_device()
+    st = _side_streams.get(key)
+    if st is None:
+        st = _side_streams[key] = torch.cuda.Stream(device=key)
+    return st
+
+
 def _launch(tag: str, info: dict, call):
     if _trace is None:
         return call()

@@ -102,6 +102,36 @@ def test_checkpointing_gives_identical_gradients():
         assert torch.equal(res[0][1][k], res[1][1][k]), k
 
 
+def test_second_stream_overlap_gives_identical_gradients():
+    """Weight / bias gradients computed on the second stream (default) against the single-stream order: the
+    kernels are deterministic, so every gradient must be bit-identical; bf16 at a size where a weight-gradient
+    GEMM spans many work-groups and uses split-K, and two backward passes so that buffers are recycled."""
+    from mi355_vit import ops
+
+    kw = dict(depth=3, hidden_size=512, intermediate_size=1200, num_heads=8, out_hidden_size=256, window_size=56, fullatt_block_indexes=[1])
+    g = torch.Generator().manual_seed(11)
+    grid = torch.tensor([[1, 32, 48], [1, 40, 28], [2, 16, 16]])
+    S = int((grid[:, 0] * grid[:, 1] * grid[:, 2]).sum())
+    pixels = torch.randn(S, 1176, generator=g)
+    gout = torch.randn(S // 4, 256, generator=g)
+    res = []
+    old = ops.OVERLAP_WGRAD
+    try:
+        for overlap in (True, False):
+            ops.OVERLAP_WGRAD = overlap
+            model = _build(kw, 7, torch.bfloat16)
+            _run_gpu(model, pixels, grid, gout)
+            for p_ in model.parameters():
+                p_.grad = None
+            res.append(_run_gpu(model, pixels, grid, gout))
+    finally:
+        ops.OVERLAP_WGRAD = old
+    assert ops.side_stream(torch.device(DEV)) is not None or not old
+    assert torch.equal(res[0][0], res[1][0])
+    for k in res[0][1]:
+        assert torch.equal(res[0][1][k], res[1][1][k]), k
+
+
 def test_reference_smoke_shape():
     """The reference's own smoke case (tests/test_ragged_sp_smoke.py:27-98): output [192, 256]."""
     kw = dict(hidden_size=256, num_heads=8, depth=2, patch_size=14, in_channels=3, out_hidden_size=256, spatial_merge_size=2,
