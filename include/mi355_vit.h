@@ -171,16 +171,19 @@ int mvit_gemm(const mvit_gemm_args* args, mvit_stream_t stream);
  * lse[h, s] = log sum exp of the scaled scores (fp32 [nheads, total]).
  * q/k/v/o element (s, h, j) lives at ptr[s*row_stride + h*head_dim + j].
  * Replaces the attention-backend call of _forward_standard, modeling:427-468 (eager: :298-321), and of
- * the sequence-parallel full-attention core, modeling:664-731 (nheads = heads / sp). */
+ * the sequence-parallel full-attention core, modeling:664-731 (nheads = heads / sp).
+ * seg_order (device, n_seg entries, may be null): a permutation of 0..n_seg-1 giving the order in which the
+ * segments are handed to the GPU.  Results do not depend on it; a work-group's run time grows with its
+ * segment's length, so listing long segments first lets the short ones fill the tail of the launch. */
 int mvit_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* cu_seqlens,
-                  int n_seg, int max_seqlen, int64_t total, int nheads, int head_dim, int64_t q_stride,
+                  const int32_t* seg_order, int n_seg, int max_seqlen, int64_t total, int nheads, int head_dim, int64_t q_stride,
                   int64_t k_stride, int64_t v_stride, int64_t o_stride, float scale, int dtype,
                   mvit_stream_t stream);
 
 /* Gradients of the above.  delta: fp32 workspace [nheads, total].  dq/dk/dv use the q/k/v strides given. */
 int mvit_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
-                  void* dq, void* dk, void* dv, float* delta, const int32_t* cu_seqlens, int n_seg,
-                  int max_seqlen, int64_t total, int nheads, int head_dim, int64_t q_stride, int64_t k_stride,
+                  void* dq, void* dk, void* dv, float* delta, const int32_t* cu_seqlens,
+                  const int32_t* seg_order, int n_seg, int max_seqlen, int64_t total, int nheads, int head_dim, int64_t q_stride, int64_t k_stride,
                   int64_t v_stride, int64_t o_stride, int64_t do_stride, int64_t dq_stride, int64_t dk_stride,
                   int64_t dv_stride, float scale, int dtype, mvit_stream_t stream);
 

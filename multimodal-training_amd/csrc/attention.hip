@@ -29,7 +29,22 @@ struct AttnParams {
   int nheads;
   int64_t q_stride, k_stride, v_stride, o_stride, do_stride, dq_stride, dk_stride, dv_stride;
   float scale;
+  const int32_t* order;  // optional: the segment scheduled at grid position i is order[i] (null: i)
+  int seg_major;         // 0: grid (x, segment, head); 1: grid (x, head, segment), all heads of a segment together
 };
+
+// Which segment and head this work-group serves.  Work per work-group grows with its segment's length, so
+// callers list long segments first: the short ones then fill the tail of the launch.
+__device__ __forceinline__ void seg_and_head(const AttnParams& p, int& seg, int& h) {
+  const int pos = p.seg_major ? blockIdx.z : blockIdx.y;
+  h = p.seg_major ? blockIdx.y : blockIdx.z;
+  seg = pos;
+  if (p.order) {
+    const int listed = p.order[pos];
+    const int n_seg = p.seg_major ? gridDim.z : gridDim.y;
+    if ((unsigned)listed < (unsigned)n_seg) seg = listed;  // an entry outside the list never becomes an address
+  }
+}
 
 typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
 typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -293,7 +308,8 @@ __global__ __launch_bounds__(64 * NWAVES, MINW) void attn_fwd_mfma(const AttnPar
   __shared__ __attribute__((aligned(16))) bf16_t lds_k[NBUF][BNK * G::PK];
   __shared__ __attribute__((aligned(16))) bf16_t lds_v[NBUF][BNK * G::PV];
 
-  const int seg = blockIdx.y, h = blockIdx.z;
+  int seg, h;
+  seg_and_head(p, seg, h);
   const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
   const int blk_q0 = blockIdx.x * (16 * QB * NWAVES);
   if (blk_q0 >= L) return;
@@ -543,7 +559,8 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
   __shared__ __attribute__((aligned(8))) bf16_t lds_fold[2][BQ][4];  // -lse2 and -delta per row, each as hi + lo
   constexpr bool FOLD = G::TAIL16;
 
-  const int seg = blockIdx.y, h = blockIdx.z;
+  int seg, h;
+  seg_and_head(p, seg, h);
   const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
   const int blk_k0 = blockIdx.x * SPAN;
   if (blk_k0 >= L) return;
@@ -714,7 +731,8 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams
   __shared__ __attribute__((aligned(16))) bf16_t lds_k[2][BK * P];
   __shared__ __attribute__((aligned(16))) bf16_t lds_v[2][BK * P];
 
-  const int seg = blockIdx.y, h = blockIdx.z;
+  int seg, h;
+  seg_and_head(p, seg, h);
   const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
   const int blk_q0 = blockIdx.x * SPAN;
   if (blk_q0 >= L) return;
@@ -853,7 +871,8 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_window_mfma(const AttnParams
   __shared__ __attribute__((aligned(16))) float lds_lse[R];
   __shared__ __attribute__((aligned(16))) float lds_delta[R];
 
-  const int seg = blockIdx.y, h = blockIdx.z;
+  int seg, h;
+  seg_and_head(p, seg, h);
   const int s0 = p.cu[seg];
   const int L = min(p.cu[seg + 1] - s0, R);
   if (L <= 0) return;
@@ -1042,7 +1061,8 @@ __global__ __launch_bounds__(64) void attn_fwd_f32(const AttnParams p) {
   constexpr int TB = 32;
   __shared__ float sk[TB * HD];
   __shared__ float sv[TB * HD];
-  const int seg = blockIdx.y, h = blockIdx.z;
+  int seg, h;
+  seg_and_head(p, seg, h);
   const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
   const int q0 = blockIdx.x * 64;
   if (q0 >= L) return;
@@ -1104,7 +1124,8 @@ __global__ __launch_bounds__(64) void attn_bwd_dq_f32(const AttnParams p) {
   constexpr int TB = 32;
   __shared__ float sk[TB * HD];
   __shared__ float sv[TB * HD];
-  const int seg = blockIdx.y, h = blockIdx.z;
+  int seg, h;
+  seg_and_head(p, seg, h);
   const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
   const int q0 = blockIdx.x * 64;
   if (q0 >= L) return;
@@ -1158,7 +1179,8 @@ __global__ __launch_bounds__(64) void attn_bwd_dkdv_f32(const AttnParams p) {
   __shared__ float sdo[TB * HD];
   __shared__ float slse[TB];
   __shared__ float sdl[TB];
-  const int seg = blockIdx.y, h = blockIdx.z;
+  int seg, h;
+  seg_and_head(p, seg, h);
   const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
   const int kb0 = blockIdx.x * 64;
   if (kb0 >= L) return;
@@ -1232,7 +1254,12 @@ int launch_fwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
   else if constexpr (ND <= 5) {
     // long segments: 8 waves x 32 queries, <= 128 registers, so that four waves share a SIMD and cover each
     // other's MFMA -> softmax -> MFMA dependency stalls
-    hipLaunchKernelGGL((attn_fwd_mfma<ND, 8, 32, true, 2, 4>), grid, 512, 0, s, p);
+    // all heads of a segment are neighbours in the launch order: with the caller's longest-first segment order
+    // the work-groups then start in order of decreasing run time
+    AttnParams pl = p;
+    pl.seg_major = 1;  // n_seg fits gridDim.z: checked at the entry point
+    dim3 gl = pl.seg_major ? dim3(grid.x, grid.z, grid.y) : grid;
+    hipLaunchKernelGGL((attn_fwd_mfma<ND, 8, 32, true, 2, 4>), gl, 512, 0, s, pl);
   }
   else hipLaunchKernelGGL((attn_fwd_mfma<ND, 4, 32, true>), grid, 256, 0, s, p);  // head_dim 128: register budget
   MVIT_CHECK_LAUNCH("attn_fwd");
@@ -1255,8 +1282,11 @@ int launch_bwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
     hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 2, 4>), grid, 128, 0, s, p);
   } else {
     dim3 grid((unsigned)((max_seqlen + 255) / 256), (unsigned)n_seg, (unsigned)p.nheads);
-    hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 8, 2>), grid, 512, 0, s, p);
-    hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 8, 2>), grid, 512, 0, s, p);
+    AttnParams pl = p;
+    pl.seg_major = 1;  // as in the forward: segment-major launch order
+    dim3 gl = pl.seg_major ? dim3(grid.x, grid.z, grid.y) : grid;
+    hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 8, 2>), gl, 512, 0, s, pl);
+    hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 8, 2>), gl, 512, 0, s, pl);
   }
   MVIT_CHECK_LAUNCH("attn_bwd");
   return MVIT_OK;
@@ -1291,15 +1321,15 @@ int check_common(const char* who, const int32_t* cu, int n_seg, int max_seqlen, 
 
 extern "C" {
 
-int mvit_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* cu_seqlens, int n_seg,
-                  int max_seqlen, int64_t total, int nheads, int head_dim, int64_t q_stride, int64_t k_stride,
+int mvit_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* cu_seqlens,
+                  const int32_t* seg_order, int n_seg, int max_seqlen, int64_t total, int nheads, int head_dim, int64_t q_stride, int64_t k_stride,
                   int64_t v_stride, int64_t o_stride, float scale, int dtype, mvit_stream_t stream) {
   if (int rc = check_common("attn_fwd", cu_seqlens, n_seg, max_seqlen, total, nheads, head_dim, dtype,
                             {q_stride, k_stride, v_stride, o_stride}, {q, k, v, o, (const void*)lse}))
     return rc;
   if (n_seg == 0 || max_seqlen == 0 || total == 0) return MVIT_OK;
   AttnParams p = {};
-  p.q = q; p.k = k; p.v = v; p.out = o; p.lse = lse; p.cu = cu_seqlens; p.total = total; p.nheads = nheads;
+  p.q = q; p.k = k; p.v = v; p.out = o; p.lse = lse; p.cu = cu_seqlens; p.order = seg_order; p.total = total; p.nheads = nheads;
   p.q_stride = q_stride; p.k_stride = k_stride; p.v_stride = v_stride; p.o_stride = o_stride; p.scale = scale;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (dtype == MVIT_BF16) {
@@ -1319,8 +1349,8 @@ int mvit_attn_fwd(const void* q, const void* k, const void* v, void* o, float* l
 }
 
 int mvit_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse, void* dq,
-                  void* dk, void* dv, float* delta, const int32_t* cu_seqlens, int n_seg, int max_seqlen, int64_t total,
-                  int nheads, int head_dim, int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
+                  void* dk, void* dv, float* delta, const int32_t* cu_seqlens, const int32_t* seg_order, int n_seg, int max_seqlen,
+                  int64_t total, int nheads, int head_dim, int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
                   int64_t do_stride, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride, float scale, int dtype,
                   mvit_stream_t stream) {
   if (int rc = check_common("attn_bwd", cu_seqlens, n_seg, max_seqlen, total, nheads, head_dim, dtype,
@@ -1330,7 +1360,7 @@ int mvit_attn_bwd(const void* q, const void* k, const void* v, const void* o, co
   if (n_seg == 0 || max_seqlen == 0 || total == 0) return MVIT_OK;
   AttnParams p = {};
   p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.lse = const_cast<float*>(lse); p.delta = delta;
-  p.dq = dq; p.dk = dk; p.dv = dv; p.cu = cu_seqlens; p.total = total; p.nheads = nheads;
+  p.dq = dq; p.dk = dk; p.dv = dv; p.cu = cu_seqlens; p.order = seg_order; p.total = total; p.nheads = nheads;
   p.q_stride = q_stride; p.k_stride = k_stride; p.v_stride = v_stride; p.o_stride = o_stride; p.do_stride = do_stride;
   p.dq_stride = dq_stride; p.dk_stride = dk_stride; p.dv_stride = dv_stride; p.scale = scale;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);

@@ -48,8 +48,8 @@ PROTOTYPES = {
     "mvit_pad_pack": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, C.c_uint32, _vp],
     "mvit_cast2d": [_vp, _i64, _i32, _vp, _i64, _i32, _i64, _i64, _vp],
     "mvit_gemm": [C.POINTER(GemmArgs), _vp],
-    "mvit_attn_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i64, _i32, _i32, _i64, _i64, _i64, _i64, _f32, _i32, _vp],
-    "mvit_attn_bwd": [_vp] * 11 + [_i32, _i32, _i64, _i32, _i32] + [_i64] * 8 + [_f32, _i32, _vp],
+    "mvit_attn_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i64, _i32, _i32, _i64, _i64, _i64, _i64, _f32, _i32, _vp],
+    "mvit_attn_bwd": [_vp] * 12 + [_i32, _i32, _i64, _i32, _i32] + [_i64] * 8 + [_f32, _i32, _vp],
 }
 EXPORTS = sorted(list(PROTOTYPES) + ["mvit_version", "mvit_last_error"])
 

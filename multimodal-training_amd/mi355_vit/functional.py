@@ -96,6 +96,7 @@ class AttnGeometry:
     head_dim: int
     cos: torch.Tensor  # fp32 [S, head_dim]
     sin: torch.Tensor
+    order: Optional[torch.Tensor] = None  # device int32 permutation of the segments, longest first (ops.segment_order)
 
 
 def _block_forward(x: torch.Tensor, W: BlockWeights, geo: AttnGeometry, eps: float) -> Tuple[torch.Tensor, tuple]:
@@ -105,7 +106,8 @@ def _block_forward(x: torch.Tensor, W: BlockWeights, geo: AttnGeometry, eps: flo
     qkv = torch.empty(S, 3 * C, dtype=x.dtype, device=x.device)
     ops.gemm(n1, W.wqkv, qkv, epilogue=E.EPI_BIAS, bias=W.bqkv.view(-1))
     ops.rope_(qkv, geo.cos, geo.sin, 2 * H, hd)  # q and k are the first 2*H heads of every row
-    o, lse = ops.attn_fwd(qkv[:, :C], qkv[:, C : 2 * C], qkv[:, 2 * C :], geo.cu, geo.max_seqlen, H, hd, hd**-0.5)
+    o, lse = ops.attn_fwd(qkv[:, :C], qkv[:, C : 2 * C], qkv[:, 2 * C :], geo.cu, geo.max_seqlen, H, hd, hd**-0.5,
+                          seg_order=geo.order)
     x1 = torch.empty_like(x)
     ops.gemm(o, W.wproj, x1, epilogue=E.EPI_BIAS_RES, bias=W.bproj.view(-1), residual=x)
     n2, rstd2 = ops.rmsnorm_fwd(x1, W.norm2.view(-1), eps)
@@ -168,7 +170,7 @@ def _block_backward(dx2: torch.Tensor, x: torch.Tensor, saved: tuple, W: BlockWe
     ops.gemm(dx1, W.wproj, d_o, trans_b=True)
     dqkv = torch.empty_like(qkv)
     ops.attn_bwd(qkv[:, :C], qkv[:, C : 2 * C], qkv[:, 2 * C :], o, d_o, lse, geo.cu, geo.max_seqlen, H, hd, hd**-0.5,
-                 dqkv[:, :C], dqkv[:, C : 2 * C], dqkv[:, 2 * C :])
+                 dqkv[:, :C], dqkv[:, C : 2 * C], dqkv[:, 2 * C :], seg_order=geo.order)
     ops.rope_(dqkv, geo.cos, geo.sin, 2 * H, hd, backward=True)
     g_bqkv = off_chain(lambda: ops.colsum(dqkv, gdt["attn.q_proj.bias"]))
     g_wqkv = torch.empty(3 * C, C, dtype=gdt["attn.q_proj.weight"], device=dev)

@@ -150,10 +150,12 @@ class Qwen2_5_VLVisionBlock(nn.Module):
                 position_embeddings = (emb.cos(), emb.sin())
             lengths = cu_seqlens[1:] - cu_seqlens[:-1]
             max_seqlen = int(lengths.max().item()) if lengths.numel() else 0  # host sync, as in the reference (:433)
+            order = ops.segment_order(lengths)
             geo = AttnGeometry(
                 cu_seqlens.to(device=hidden_states.device, dtype=torch.int32).contiguous(), max_seqlen,
                 self.attn.num_heads, self.attn.head_dim,
                 position_embeddings[0].float().contiguous(), position_embeddings[1].float().contiguous(),
+                None if order is None else order.to(hidden_states.device),
             )
         ckpt = self.gradient_checkpointing and self.training and torch.is_grad_enabled()
         return VisionBlockFn.apply(hidden_states, self, geo, self.norm1.variance_epsilon, ckpt, *self._block_params())
@@ -182,6 +184,9 @@ class _TowerPlan:
         self.cu_window, self.cu_full = cu_w.to(device), cu_f.to(device)
         self.max_window = int((cu_w[1:] - cu_w[:-1]).max()) if cu_w.numel() > 1 else 0
         self.max_full = int((cu_f[1:] - cu_f[:-1]).max()) if cu_f.numel() > 1 else 0
+        order_w, order_f = ops.segment_order(cu_w[1:] - cu_w[:-1]), ops.segment_order(cu_f[1:] - cu_f[:-1])
+        self.order_window = None if order_w is None else order_w.to(device)
+        self.order_full = None if order_f is None else order_f.to(device)
 
 
 class Qwen2_5_VisionTransformerPretrainedModel(nn.Module):
@@ -291,8 +296,8 @@ class Qwen2_5_VisionTransformerPretrainedModel(nn.Module):
         cos, sin = emb.cos().float().contiguous(), emb.sin().float().contiguous()
 
         H, hd = self.config.num_heads, self.config.hidden_size // self.config.num_heads
-        geo_full = AttnGeometry(plan.cu_full, plan.max_full, H, hd, cos, sin)
-        geo_win = AttnGeometry(plan.cu_window, plan.max_window, H, hd, cos, sin)
+        geo_full = AttnGeometry(plan.cu_full, plan.max_full, H, hd, cos, sin, plan.order_full)
+        geo_win = AttnGeometry(plan.cu_window, plan.max_window, H, hd, cos, sin, plan.order_window)
         for layer_num, blk in enumerate(self.blocks):
             full = layer_num in self.fullatt_block_indexes
             x = blk(x, cu_seqlens=plan.cu_full if full else plan.cu_window, position_embeddings=(cos, sin),

@@ -392,8 +392,28 @@ def _attn_view(t: torch.Tensor, nheads: int, head_dim: int, what: str) -> int:
     return t.stride(0)
 
 
-def attn_fwd(q, k, v, cu_seqlens: torch.Tensor, max_seqlen: int, nheads: int, head_dim: int, scale: float, out: Optional[torch.Tensor] = None):
-    """q, k, v: [S, nheads*head_dim] views (row strides free).  Returns (o [S, nheads*head_dim], lse [nheads, S])."""
+def segment_order(lengths: torch.Tensor) -> Optional[torch.Tensor]:
+    """int32 permutation of the segments, longest first (stable), for the ``seg_order`` argument of the attention
+    calls; None when all segments that matter are equally long (the natural order is then as good).  Host tensor in,
+    host tensor out."""
+    ln = lengths.detach().to("cpu", torch.int64)
+    if ln.numel() < 2 or int(ln.max()) <= 64:  # windows: one work-group each, all alike
+        return None
+    return torch.sort(ln, descending=True, stable=True).indices.to(torch.int32).contiguous()
+
+
+def _order_ptr(seg_order: Optional[torch.Tensor], cu_seqlens: torch.Tensor) -> Optional[int]:
+    if seg_order is None:
+        return None
+    if seg_order.dtype != torch.int32 or seg_order.device != cu_seqlens.device or not seg_order.is_contiguous() or seg_order.numel() != cu_seqlens.numel() - 1:
+        raise ValueError("attn: seg_order must be a contiguous int32 permutation of the segments on the inputs' device")
+    return seg_order.data_ptr()
+
+
+def attn_fwd(q, k, v, cu_seqlens: torch.Tensor, max_seqlen: int, nheads: int, head_dim: int, scale: float, out: Optional[torch.Tensor] = None,
+             seg_order: Optional[torch.Tensor] = None):
+    """q, k, v: [S, nheads*head_dim] views (row strides free).  Returns (o [S, nheads*head_dim], lse [nheads, S]).
+    ``seg_order``: optional scheduling order of the segments (see segment_order); results do not depend on it."""
     S = q.shape[0]
     if cu_seqlens.dtype != torch.int32 or cu_seqlens.device != q.device or not cu_seqlens.is_contiguous():
         raise ValueError("attn: cu_seqlens must be a contiguous int32 tensor on the inputs' device")
@@ -402,18 +422,20 @@ def attn_fwd(q, k, v, cu_seqlens: torch.Tensor, max_seqlen: int, nheads: int, he
     if out is None:
         out = torch.empty(S, nheads * head_dim, dtype=q.dtype, device=q.device)
     lse = torch.empty(nheads, S, dtype=torch.float32, device=q.device)
+    order_ptr = _order_ptr(seg_order, cu_seqlens)
     st = _stream(q)
     strides = (_attn_view(q, nheads, head_dim, "attn q"), _attn_view(k, nheads, head_dim, "attn k"),
                _attn_view(v, nheads, head_dim, "attn v"), _attn_view(out, nheads, head_dim, "attn o"))
     rc = _launch("attn_fwd", {"cu": cu_seqlens, "max_seqlen": max_seqlen, "nheads": nheads, "head_dim": head_dim}, lambda: _lib.load().mvit_attn_fwd(
-        q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), cu_seqlens.data_ptr(),
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), cu_seqlens.data_ptr(), order_ptr,
         cu_seqlens.numel() - 1, max_seqlen, S, nheads, head_dim, *strides, scale, dt(q), st))
     _lib.check(rc, "mvit_attn_fwd")
     return out, lse
 
 
-def attn_bwd(q, k, v, o, d_o, lse, cu_seqlens, max_seqlen, nheads, head_dim, scale, dq, dk, dv):
+def attn_bwd(q, k, v, o, d_o, lse, cu_seqlens, max_seqlen, nheads, head_dim, scale, dq, dk, dv, seg_order: Optional[torch.Tensor] = None):
     """Writes dq, dk, dv ([S, nheads*head_dim] views, row strides free)."""
+    order_ptr = _order_ptr(seg_order, cu_seqlens)
     S = q.shape[0]
     for t in (k, v, o, d_o, dq, dk, dv):
         if t.shape[0] != S or t.dtype != q.dtype:
@@ -425,7 +447,7 @@ def attn_bwd(q, k, v, o, d_o, lse, cu_seqlens, max_seqlen, nheads, head_dim, sca
     strides = tuple(_attn_view(t, nheads, head_dim, nm) for t, nm in ((q, "q"), (k, "k"), (v, "v"), (o, "o"), (d_o, "do"), (dq, "dq"), (dk, "dk"), (dv, "dv")))
     rc = _launch("attn_bwd", {"cu": cu_seqlens, "max_seqlen": max_seqlen, "nheads": nheads, "head_dim": head_dim}, lambda: _lib.load().mvit_attn_bwd(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(), lse.data_ptr(),
-        dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(), cu_seqlens.data_ptr(),
+        dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(), cu_seqlens.data_ptr(), order_ptr,
         cu_seqlens.numel() - 1, max_seqlen, S, nheads, head_dim, *strides, scale, dt(q), st))
     _lib.check(rc, "mvit_attn_bwd")
     return dq, dk, dv

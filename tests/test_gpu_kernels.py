@@ -397,6 +397,40 @@ def test_attention_long_segment_bf16():
     _attn_case(torch.bfloat16, [2048, 1000], 4, 80, qkv_packed=False)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_segment_order_changes_nothing(dtype):
+    """seg_order only changes which work-group serves which segment: outputs and gradients are bit-identical with
+    the natural order, the longest-first order of ops.segment_order and an arbitrary permutation; long (multi-block)
+    and window-sized layouts."""
+    ops = _ops()
+    H, d = 4, 80
+    for seglens in ([300, 1200, 77, 640, 1, 513], [64, 16, 48, 64]):
+        _announce(f"attention seg_order {dtype} {seglens}")
+        S = sum(seglens)
+        cu = torch.tensor([0] + list(np.cumsum(seglens)), dtype=torch.int32).to(DEV)
+        qkv = _rand((S, 3 * H * d), dtype, 5).to(DEV)
+        q, k, v = qkv[:, : H * d], qkv[:, H * d : 2 * H * d], qkv[:, 2 * H * d :]
+        do = _rand((S, H * d), dtype, 6).to(DEV)
+        lf = ops.segment_order(torch.tensor(seglens))
+        if max(seglens) > 64:
+            assert lf.tolist() == sorted(range(len(seglens)), key=lambda i: -seglens[i])
+        else:
+            assert lf is None
+        orders = [None, lf, torch.tensor(list(range(len(seglens)))[::-1], dtype=torch.int32)]
+        res = []
+        for order in orders:
+            od = None if order is None else order.to(DEV)
+            o, lse = ops.attn_fwd(q, k, v, cu, max(seglens), H, d, d**-0.5, seg_order=od)
+            dq, dk, dv = (torch.full((S, H * d), float("nan"), dtype=dtype, device=DEV) for _ in range(3))
+            ops.attn_bwd(q, k, v, o, do, lse, cu, max(seglens), H, d, d**-0.5, dq, dk, dv, seg_order=od)
+            res.append((o, lse, dq, dk, dv))
+        for other in res[1:]:
+            for a, b in zip(res[0], other):
+                assert torch.equal(a, b)
+    with pytest.raises(ValueError):
+        ops.attn_fwd(q, k, v, cu, 64, H, d, d**-0.5, seg_order=torch.zeros(2, dtype=torch.int32, device=DEV))
+
+
 def test_attention_sp_share_real_shape():
     """One rank's share of Ulysses SP=4 attention at its real shape: 65,536 tokens, 4 of the 16 heads, head_dim 80.
     Windowed layout (64-token windows): everything against the oracle.  Full layer: the oracle's O(L^2) pass is
