@@ -109,7 +109,7 @@ KERNEL_NAMES = {
     "attn_fwd_full": "attn_fwd_mfma<5, 8, 32, true, 2, 4>",
     "attn_bwd_full": "attn_delta_kernel + attn_bwd_dkdv_mfma<5, 8, 2> + attn_bwd_dq_mfma<5, 8, 2>",
     "attn_fwd_window": "attn_fwd_mfma<5, 2, 64, false, 2, 4>",
-    "attn_bwd_window": "attn_bwd_window_mfma<5, 2>",
+    "attn_bwd_window": "attn_bwd_window_mfma<5, 4, 2>",
 }
 
 

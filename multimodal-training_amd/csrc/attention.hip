@@ -860,8 +860,8 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams
 // (segment, head) are staged in LDS once.  Pass A works in the dQ orientation (a lane owns a query), where
 // delta_q = sum_k P[q,k] * dP[q,k] (equal to dO_q . O_q, so O is never read) is a lane-local sum, and writes dQ;
 // pass B repeats the dK/dV kernel's tile loop on the staged tiles.  HBM traffic: four tiles in, three out.
-template <int ND, int NW>  // NW waves share the staged tiles; wave w owns query / key blocks [w*4/NW, (w+1)*4/NW)
-__global__ __launch_bounds__(64 * NW) void attn_bwd_window_mfma(const AttnParams p) {
+template <int ND, int NW, int MINW = 1>  // NW waves share the staged tiles; wave w owns query / key blocks [w*4/NW, (w+1)*4/NW)
+__global__ __launch_bounds__(64 * NW, MINW) void attn_bwd_window_mfma(const AttnParams p) {
   using G = Geo<ND>;
   constexpr int HD = G::HD, R = 64, PK = G::PK, NB = 4 / NW;  // NB 16-row blocks per wave
   __shared__ __attribute__((aligned(16))) bf16_t lds_q[R * PK];
@@ -1271,7 +1271,8 @@ int launch_bwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
   if (max_seqlen <= 64) {
     dim3 grid(1, (unsigned)n_seg, (unsigned)p.nheads);
     if constexpr (ND <= 5) {
-      hipLaunchKernelGGL((attn_bwd_window_mfma<ND, 2>), grid, 128, 0, s, p);  // computes delta itself
+      // four waves x 16 rows: ~160 registers, three work-groups (12 waves) per CU to cover the load -> MFMA -> store latency
+      hipLaunchKernelGGL((attn_bwd_window_mfma<ND, 4, 2>), grid, 256, 0, s, p);  // computes delta itself
     } else {
       hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 1, 4>), grid, 64, 0, s, p);
       hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 1, 4>), grid, 64, 0, s, p);
