@@ -113,6 +113,48 @@ KERNEL_NAMES = {
 }
 
 
+def optimizer_leg(model, step, iters: int = 5):
+    """The step after the path (not part of `value`): gradient norm, clipping and Adam over every parameter tensor.
+    Multi-tensor kernels (one launch each) against what the reference calls on the same GPU: torch.optim.Adam(
+    foreach=False) after a per-tensor gradient-scaling loop, and the per-tensor norm(2).item() loop."""
+    from mi355_vit.optim import FusedAdam, grad_norm_squared
+
+    params = [p for p in model.parameters() if p.requires_grad]
+    n = sum(p.numel() for p in params)
+    esize = params[0].element_size()
+    step()  # fresh gradients
+    torch.cuda.synchronize()
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return 1000.0 * (time.perf_counter() - t0) / reps
+
+    fused = FusedAdam(params, lr=1e-5)
+    fused_ms = timed(lambda: fused.step(grad_scale=0.5), iters)
+    norm_ms = timed(lambda: grad_norm_squared(params), iters)
+    del fused
+    ref = torch.optim.Adam(params, lr=1e-5, foreach=False)
+
+    def ref_step():
+        for p in params:
+            p.grad.mul_(0.5)
+        ref.step()
+
+    ref_ms = timed(ref_step, 2)
+    ref_norm_ms = timed(lambda: sum(p.grad.float().norm(2).item() ** 2 for p in params), 2)
+    del ref
+    traffic = n * esize * 8  # read p, g, m, v; write p, g (scaled), m, v
+    return {"tensors": len(params), "parameters": n, "dtype": str(params[0].dtype).replace("torch.", ""),
+            "adam_with_clip_ms": round(fused_ms, 3), "adam_with_clip_gbs": round(traffic / (fused_ms * 1e-3) / 1e9, 1),
+            "grad_norm_ms": round(norm_ms, 3), "grad_norm_gbs": round(n * esize / (norm_ms * 1e-3) / 1e9, 1),
+            "torch_adam_foreach_false_with_clip_ms": round(ref_ms, 3), "torch_norm_loop_ms": round(ref_norm_ms, 3)}
+
+
 def cpu_baseline(cfg_kw, grid, seed, dtype, budget_s: float = 25.0):
     """Eager oracle (the reference's per-segment path, fp32) on the host cores, on a bounded sample: the two
     smallest images of the batch through patch embed, one windowed and one full-attention block and the
@@ -170,6 +212,7 @@ def main() -> None:
     ap.add_argument("--single-stream", action="store_true",
                     help="run weight / bias gradients in line on the main stream instead of on the second stream (for profiler "
                          "runs: kernels then never share the GPU, so their traced durations are their own)")
+    ap.add_argument("--no-optimizer", action="store_true", help="skip the optimizer-step measurement (reported beside the metric, never inside it)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain device copy of 1 GiB (8 launches) so that profiler byte counters can be scaled to a known size")
     args = ap.parse_args()
@@ -249,6 +292,10 @@ def main() -> None:
                 e["gbs"] = round(v["bytes"] / (v["ms"] * 1e-3) / 1e9, 1)
             breakdown[k] = e
 
+    optimizer = None
+    if not args.no_optimizer:
+        optimizer = optimizer_leg(model, step)
+
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(cfg_kw, grid, seed, dtype)
@@ -272,6 +319,7 @@ def main() -> None:
         "attention_mfma_util": attn_util,
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "optimizer_step": optimizer,
         "kernel_breakdown": breakdown,
     }
     print(json.dumps(result))

@@ -187,6 +187,49 @@ int mvit_attn_bwd(const void* q, const void* k, const void* v, const void* o, co
                   int64_t v_stride, int64_t o_stride, int64_t do_stride, int64_t dq_stride, int64_t dk_stride,
                   int64_t dv_stride, float scale, int dtype, mvit_stream_t stream);
 
+/* ---------------------------------------------------------------- optimizer step (multi-tensor) */
+
+#define MVIT_ADAM_CHUNK 8192 /* elements per work-group; a chunk never spans two tensors */
+
+/* One parameter tensor of a multi-tensor launch.  The table lives in DEVICE memory and has n_tensors + 1
+ * entries: entry i covers chunks [first_chunk(i), first_chunk(i+1)), first_chunk(i+1) - first_chunk(i) =
+ * ceil(numel(i) / MVIT_ADAM_CHUNK), first_chunk(0) = 0, and the last entry is a sentinel whose first_chunk
+ * is the total chunk count (its other fields are ignored).  The kernels trust the table.
+ * step_size = lr / (1 - beta1^step) and bias_correction2_sqrt = sqrt(1 - beta2^step) are computed by the
+ * caller in double precision, as torch/optim/adam.py does on the host. */
+typedef struct {
+  void* param;       /* [numel] dtype, updated in place */
+  void* grad;        /* [numel] dtype; rewritten with grad * grad_scale when write_grad != 0 */
+  void* exp_avg;     /* [numel] dtype, first moment */
+  void* exp_avg_sq;  /* [numel] dtype, second moment */
+  int64_t numel;
+  int64_t first_chunk;
+  float step_size;
+  float bias_correction2_sqrt;
+  float weight_decay; /* L2 term: grad + weight_decay * param, as torch.optim.Adam (not decoupled) */
+  float reserved;
+} mvit_adam_tensor;
+
+/* torch.optim.Adam(foreach=False, amsgrad=False, maximize=False) for every tensor of the table in one launch:
+ *   g = grad * grad_scale; g += weight_decay * p; m += (1 - beta1) (g - m); v = v beta2 + (1 - beta2) g g;
+ *   p -= step_size * m / (sqrt(v) / bias_correction2_sqrt + eps)
+ * one operation at a time in fp32, each result rounded to `dtype` when that is bf16 (what the per-tensor
+ * torch kernels do).  grad_scale is the clipping coefficient of Trainer._clip_gradients (1 = none); with
+ * write_grad the scaled gradient is stored back, as the reference's in-place grad.mul_ leaves it.
+ * The hyper-parameters are doubles (Python floats): 1 - beta1 and 1 - beta2 are formed in double and rounded
+ * to fp32 once, as they reach torch's kernels.
+ * Replaces Trainer.optimizer_step -> self.optimizer.step() (trainer.py:158-189, optimizer built at :479-577)
+ * and the scaling loop of Trainer._clip_gradients (trainer.py:123-156). */
+int mvit_adam_step(const mvit_adam_tensor* tensors, int n_tensors, int64_t n_chunks, double beta1, double beta2,
+                   double eps, double grad_scale, int write_grad, int dtype, mvit_stream_t stream);
+
+/* out[0] (fp64, device) = sum over all tensors of the table of sum(grad^2): only `grad`, `numel` and
+ * `first_chunk` of each entry are read.  partial: fp32 workspace [n_chunks].  Replaces the per-tensor
+ * norm(2).item() ** 2 loop of Trainer._compute_grad_norm_squared (trainer.py:293-308) with two launches
+ * and one read-back by the caller. */
+int mvit_grad_sumsq(const mvit_adam_tensor* tensors, int n_tensors, int64_t n_chunks, float* partial, double* out,
+                    int dtype, mvit_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

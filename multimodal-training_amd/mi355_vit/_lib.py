@@ -31,6 +31,18 @@ class GemmArgs(C.Structure):
     ]
 
 
+class AdamTensor(C.Structure):
+    """mvit_adam_tensor: one row of the device-resident tensor table of the multi-tensor optimizer kernels."""
+
+    _fields_ = [
+        ("param", _vp), ("grad", _vp), ("exp_avg", _vp), ("exp_avg_sq", _vp),
+        ("numel", _i64), ("first_chunk", _i64),
+        ("step_size", _f32), ("bias_correction2_sqrt", _f32), ("weight_decay", _f32), ("reserved", _f32),
+    ]
+
+
+ADAM_CHUNK = 8192
+
 # name -> argument types (every function returns int except the two noted below)
 PROTOTYPES = {
     "mvit_rot_pos_ids": [_vp, _i64, _i32, _vp],
@@ -49,6 +61,8 @@ PROTOTYPES = {
     "mvit_cast2d": [_vp, _i64, _i32, _vp, _i64, _i32, _i64, _i64, _vp],
     "mvit_gemm": [C.POINTER(GemmArgs), _vp],
     "mvit_attn_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i64, _i32, _i32, _i64, _i64, _i64, _i64, _f32, _i32, _vp],
+    "mvit_adam_step": [_vp, _i32, _i64, C.c_double, C.c_double, C.c_double, C.c_double, _i32, _i32, _vp],
+    "mvit_grad_sumsq": [_vp, _i32, _i64, _vp, _vp, _i32, _vp],
     "mvit_attn_bwd": [_vp] * 12 + [_i32, _i32, _i64, _i32, _i32] + [_i64] * 8 + [_f32, _i32, _vp],
 }
 EXPORTS = sorted(list(PROTOTYPES) + ["mvit_version", "mvit_last_error"])

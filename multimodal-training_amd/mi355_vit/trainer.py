@@ -31,6 +31,7 @@ import torch
 
 from .config import Qwen2_5_VLVisionConfig
 from .modeling import Qwen2_5_VisionTransformerPretrainedModel
+from .optim import FusedAdam, grad_norm_squared
 
 logger = logging.getLogger(__name__)
 
@@ -94,11 +95,23 @@ class Trainer:
                         p.grad.mul_(clip_coeff)
         return clip_coeff
 
+    def _optimizer_covers_trainables(self) -> bool:
+        owned = {id(p) for group in self.optimizer.param_groups for p in group["params"]}
+        return all(id(p) in owned for _, mod in self._trainable_modules() for p in mod.parameters() if p.grad is not None)
+
     def optimizer_step(self, global_grad_norm: Optional[float] = None) -> float:
         clip_coeff = 1.0
+        in_step_scale = 1.0
         if global_grad_norm is not None:
-            clip_coeff = self._clip_gradients(global_grad_norm, self.config.get("max_grad_norm", 1.0))
-        if self.optimizer is not None:
+            max_norm = self.config.get("max_grad_norm", 1.0)
+            if isinstance(self.optimizer, FusedAdam) and self._optimizer_covers_trainables():
+                # the multi-tensor step scales the gradients itself (and stores them back scaled): one pass instead of two
+                clip_coeff = in_step_scale = min(1.0, max_norm / (global_grad_norm + 1e-6))
+            else:
+                clip_coeff = self._clip_gradients(global_grad_norm, max_norm)
+        if isinstance(self.optimizer, FusedAdam):
+            self.optimizer.step(grad_scale=in_step_scale)
+        elif self.optimizer is not None:
             self.optimizer.step()
         if self.scheduler is not None:
             self.scheduler.step()
@@ -113,10 +126,12 @@ class Trainer:
                 p.grad = None
 
     def _compute_grad_norm_squared(self, params) -> float:
+        params = [p for p in params if p.grad is not None]
+        if params and all(p.grad.is_cuda for p in params):
+            return grad_norm_squared(params)  # two launches and one read-back for all tensors
         total = 0.0
-        for p in params:
-            if p.grad is not None:
-                total += p.grad.detach().float().norm(2).item() ** 2
+        for p in params:  # host tensors (no GPU work to save)
+            total += p.grad.detach().float().norm(2).item() ** 2
         return total
 
     def compute_grad_norm_contribution(self) -> dict:
@@ -141,8 +156,11 @@ class Trainer:
             return
         lr = self.config["learning_rate"] if learning_rate is None else learning_rate
         wd = self.config["weight_decay"]
+        # parameters on the GPU (always, once build_model has run) get the multi-tensor step; the class is a
+        # torch.optim.Adam with the same groups and state, so schedulers and checkpoints do not see a difference
+        Adam = FusedAdam if all(p.is_cuda for p in plist) else torch.optim.Adam
         if wd == 0.0:
-            self.optimizer = torch.optim.Adam(plist, lr=lr, foreach=False)
+            self.optimizer = Adam(plist, lr=lr, foreach=False)
             return
         named, seen = [], set()
         for mname, mod in self._trainable_modules():
@@ -151,12 +169,12 @@ class Trainer:
                     named.append((f"{mname}.{n}", p))
                     seen.add(id(p))
         if not named:
-            self.optimizer = torch.optim.Adam(plist, lr=lr, foreach=False)
+            self.optimizer = Adam(plist, lr=lr, foreach=False)
             return
         decay_names = self._get_decay_parameter_names(named)
         decay = [p for n, p in named if p.requires_grad and n in decay_names]
         no_decay = [p for n, p in named if p.requires_grad and n not in decay_names]
-        self.optimizer = torch.optim.Adam(
+        self.optimizer = Adam(
             [{"params": decay, "weight_decay": wd}, {"params": no_decay, "weight_decay": 0.0}], lr=lr, foreach=False)
 
     def _build_scheduler(self, num_training_steps: int) -> None:
