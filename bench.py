@@ -155,6 +155,56 @@ def optimizer_leg(model, step, iters: int = 5):
             "torch_adam_foreach_false_with_clip_ms": round(ref_ms, 3), "torch_norm_loop_ms": round(ref_norm_ms, 3)}
 
 
+def handoff_leg(n_vision: int, hidden: int, dtype, iters: int = 20):
+    """The step after the tower's output (not part of `value`): the [M, O] embeddings go into the <image> slots of a
+    text sequence of M + 1024 tokens and the slot gradients come back.  Ranking + row-merge kernels against the
+    reference's own calls on the same GPU (three counting guards with read-backs, masked_scatter, autograd)."""
+    from mi355_vit.handoff import IMAGE_TOKEN_ID, extract_vision_grad, merge_vision_embeddings, prepare_vision_embeddings
+
+    dev = torch.device("cuda:0")
+    T = n_vision + 1024
+    g = torch.Generator().manual_seed(0)
+    ids = torch.randint(0, 1000, (1, T), generator=g)
+    ids[0, 512 : 512 + n_vision] = IMAGE_TOKEN_ID
+    labels = torch.randint(0, 1000, (1, T), generator=g)
+    labels[ids == IMAGE_TOKEN_ID] = -100
+    ids, labels = ids.to(dev), labels.to(dev)
+    text = torch.randn(1, T, hidden, generator=g).to(dev, dtype).requires_grad_(True)
+    vis = torch.randn(n_vision, hidden, generator=g).to(dev, dtype)
+    gout = torch.randn(1, T, hidden, generator=g).to(dev, dtype)
+
+    def ours():
+        leaf = prepare_vision_embeddings(vis)
+        merge_vision_embeddings(text, ids, leaf, labels).backward(gout)
+        text.grad = None
+        return extract_vision_grad(leaf)
+
+    def reference_calls():
+        leaf = prepare_vision_embeddings(vis)
+        mask = (ids == IMAGE_TOKEN_ID).unsqueeze(-1).expand_as(text)
+        n = (ids == IMAGE_TOKEN_ID).sum().item()
+        assert n == leaf.shape[1] and bool(torch.all(labels[ids == IMAGE_TOKEN_ID] == -100))
+        text.masked_scatter(mask, leaf.reshape(-1, hidden)).backward(gout)
+        text.grad = None
+        return extract_vision_grad(leaf)
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            fn()
+        torch.cuda.synchronize()
+        return 1000.0 * (time.perf_counter() - t0) / iters
+
+    assert torch.equal(ours(), reference_calls())
+    ours_ms, ref_ms = timed(ours), timed(reference_calls)
+    esize = text.element_size()
+    moved = (4 * T * hidden + 2 * n_vision * hidden) * esize  # merge fwd, zero-filling merge bwd, row gather bwd
+    return {"tokens": T, "vision_rows": n_vision, "hidden": hidden, "fwd_bwd_ms": round(ours_ms, 3),
+            "kernel_bytes_gbs": round(moved / (ours_ms * 1e-3) / 1e9, 1), "torch_masked_scatter_fwd_bwd_ms": round(ref_ms, 3)}
+
+
 def cpu_baseline(cfg_kw, grid, seed, dtype, budget_s: float = 25.0):
     """Eager oracle (the reference's per-segment path, fp32) on the host cores, on a bounded sample: the two
     smallest images of the batch through patch embed, one windowed and one full-attention block and the
@@ -296,6 +346,10 @@ def main() -> None:
     if not args.no_optimizer:
         optimizer = optimizer_leg(model, step)
 
+    handoff = None
+    if not args.no_optimizer:
+        handoff = handoff_leg(S // 4, cfg_kw["out_hidden_size"], dtype)
+
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(cfg_kw, grid, seed, dtype)
@@ -320,6 +374,7 @@ def main() -> None:
         "roofline": roofline,
         "cpu_baseline": cpu,
         "optimizer_step": optimizer,
+        "vision_text_handoff": handoff,
         "kernel_breakdown": breakdown,
     }
     print(json.dumps(result))

@@ -87,7 +87,7 @@ int mvit_reduce_partials(const float* partial, int n_partial, int64_t cols, void
 int mvit_rope(void* x, const float* cos, const float* sin, int64_t rows, int nheads, int head_dim,
               int64_t row_stride, int backward, int dtype, mvit_stream_t stream);
 
-/* dst[i, :] = src[index[i], :] for rows of row_bytes bytes (multiple of 4).  Bit-exact.
+/* dst[i, :] = src[index[i], :] for rows of row_bytes bytes (multiple of 2).  Bit-exact.
  * Replaces the window reorder x.view(M,4,C)[window_index] and its inverse, modeling:934-940, :1067-1068. */
 int mvit_gather_rows(const void* src, const int64_t* index, void* dst, int64_t n_rows, int64_t row_bytes,
                      mvit_stream_t stream);
@@ -186,6 +186,25 @@ int mvit_attn_bwd(const void* q, const void* k, const void* v, const void* o, co
                   const int32_t* seg_order, int n_seg, int max_seqlen, int64_t total, int nheads, int head_dim, int64_t q_stride, int64_t k_stride,
                   int64_t v_stride, int64_t o_stride, int64_t do_stride, int64_t dq_stride, int64_t dk_stride,
                   int64_t dv_stride, float scale, int dtype, mvit_stream_t stream);
+
+/* ---------------------------------------------------------------- vision -> text hand-off */
+
+/* Ranks the image placeholders of a token sequence: rank[t] = k (0-based) if input_ids[t] is the k-th entry equal
+ * to image_token_id, else -1; positions[k] = t; counts[0] = number of placeholders; counts[1] = number of
+ * placeholders whose label differs from ignore_label (0 when labels is null).  All device pointers; rank
+ * [n_tokens] int32, positions [n_tokens] int64 (first counts[0] entries written), counts [2] int64.
+ * Replaces the mask building and the counting guards of TextTrainer's forward, python/ray/text.py:883-910. */
+int mvit_image_token_ranks(const int64_t* input_ids, const int64_t* labels, int64_t n_tokens, int64_t image_token_id,
+                           int64_t ignore_label, int32_t* rank, int64_t* positions, int64_t* counts,
+                           mvit_stream_t stream);
+
+/* merged[t, :] = rank[t] >= 0 ? vision[rank[t], :] : embeds[t, :] over rows of row_bytes bytes (bit-exact copy);
+ * with vision == NULL the selected rows are zero-filled instead.  A rank >= n_vision keeps the embeds row.
+ * Forward: inputs_embeds.masked_scatter(image_mask, vision_embeds_flat), python/ray/text.py:913.  Backward: the
+ * gradient of the text rows is mvit_merge_rows(grad, NULL, ...) and the gradient handed back to the vision actor
+ * (text.py:1000-1019) is mvit_gather_rows(grad, positions, ...). */
+int mvit_merge_rows(const void* embeds, const void* vision, const int32_t* rank, void* merged, int64_t n_tokens,
+                    int64_t n_vision, int64_t row_bytes, mvit_stream_t stream);
 
 /* ---------------------------------------------------------------- optimizer step (multi-tensor) */
 

@@ -331,6 +331,67 @@ __global__ __launch_bounds__(256) void cast2d_kernel(const S* __restrict__ src, 
 
 // ------------------------------------------------------------------------------------------------
 static inline hipStream_t S_(mvit_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+// ------------------------------------------------------------------------------------------------
+// Vision -> text hand-off: where the token ids equal the image placeholder, the rows of the text embedding are
+// replaced by the vision rows, the k-th placeholder taking vision row k (masked_scatter with a row mask).
+// One work-group ranks the placeholders (each thread counts a contiguous slice, the counts are scanned in LDS, the
+// slice is walked again to write ranks and positions); the row merge is then a pure byte copy.
+__global__ __launch_bounds__(1024) void image_token_ranks_kernel(const int64_t* __restrict__ ids, const int64_t* __restrict__ labels,
+                                                                 int64_t n, int64_t image_id, int64_t ignore_label,
+                                                                 int32_t* __restrict__ rank, int64_t* __restrict__ positions,
+                                                                 int64_t* __restrict__ counts) {
+  __shared__ int scan[1024];
+  __shared__ int bad[1024];
+  const int t = threadIdx.x;
+  const int64_t per = (n + 1023) / 1024;
+  const int64_t lo = per * t < n ? per * t : n;
+  const int64_t hi = lo + per < n ? lo + per : n;
+  int cnt = 0, wrong = 0;
+  for (int64_t i = lo; i < hi; ++i) {
+    const bool img = ids[i] == image_id;
+    cnt += img;
+    if (img && labels != nullptr && labels[i] != ignore_label) ++wrong;
+  }
+  scan[t] = cnt;
+  bad[t] = wrong;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {  // inclusive scan (Hillis-Steele), and a plain sum for the label check
+    const int v = t >= off ? scan[t - off] : 0;
+    const int w = t >= off ? bad[t - off] : 0;
+    __syncthreads();
+    scan[t] += v;
+    bad[t] += w;
+    __syncthreads();
+  }
+  int k = scan[t] - cnt;  // exclusive prefix of this slice
+  for (int64_t i = lo; i < hi; ++i) {
+    if (ids[i] == image_id) {
+      rank[i] = k;
+      positions[k] = i;
+      ++k;
+    } else {
+      rank[i] = -1;
+    }
+  }
+  if (t == 1023) {
+    counts[0] = scan[1023];
+    counts[1] = bad[1023];
+  }
+}
+
+template <typename W>
+__global__ __launch_bounds__(256) void merge_rows_kernel(const W* __restrict__ embeds, const W* __restrict__ vision,
+                                                         const int32_t* __restrict__ rank, W* __restrict__ merged, int64_t n_rows,
+                                                         int64_t n_vision, int64_t row_words) {
+  for (int64_t r = blockIdx.y; r < n_rows; r += gridDim.y) {
+    const int k = rank[r];
+    const bool img = k >= 0 && k < n_vision;  // a rank beyond the vision rows keeps the text row (the caller has refused that case)
+    const W* s = img ? (vision ? vision + (int64_t)k * row_words : nullptr) : embeds + r * row_words;
+    W* d = merged + r * row_words;
+    for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < row_words; c += (int64_t)gridDim.x * 256) d[c] = s ? s[c] : W{};
+  }
+}
+
 static inline int clamp_grid(int64_t v, int64_t hi) { return (int)(v < 1 ? 1 : (v > hi ? hi : v)); }
 
 extern "C" {
@@ -461,17 +522,21 @@ int mvit_rope(void* x, const float* cosb, const float* sinb, int64_t rows, int n
 
 int mvit_gather_rows(const void* src, const int64_t* index, void* dst, int64_t n_rows, int64_t row_bytes, mvit_stream_t stream) {
   MVIT_REQUIRE(src && index && dst, "gather_rows: null pointer");
-  MVIT_REQUIRE(n_rows >= 0 && row_bytes > 0 && row_bytes % 4 == 0, "gather_rows: row_bytes %lld must be a positive multiple of 4", (long long)row_bytes);
+  MVIT_REQUIRE(n_rows >= 0 && row_bytes > 0 && row_bytes % 2 == 0, "gather_rows: row_bytes %lld must be a positive multiple of 2", (long long)row_bytes);
   if (n_rows == 0) return MVIT_OK;
   const unsigned gy = (unsigned)clamp_grid(n_rows, 65535);
   if (row_bytes % 16 == 0 && mvit_aligned16(src) && mvit_aligned16(dst)) {
     const int64_t words = row_bytes / 16;
     dim3 grid((unsigned)clamp_grid((words + 255) / 256, 64), gy);
     hipLaunchKernelGGL((gather_rows_kernel<u32x4>), grid, 256, 0, S_(stream), (const u32x4*)src, index, (u32x4*)dst, n_rows, words);
-  } else {
+  } else if (row_bytes % 4 == 0) {
     const int64_t words = row_bytes / 4;
     dim3 grid((unsigned)clamp_grid((words + 255) / 256, 64), gy);
     hipLaunchKernelGGL((gather_rows_kernel<uint32_t>), grid, 256, 0, S_(stream), (const uint32_t*)src, index, (uint32_t*)dst, n_rows, words);
+  } else {
+    const int64_t words = row_bytes / 2;
+    dim3 grid((unsigned)clamp_grid((words + 255) / 256, 64), gy);
+    hipLaunchKernelGGL((gather_rows_kernel<uint16_t>), grid, 256, 0, S_(stream), (const uint16_t*)src, index, (uint16_t*)dst, n_rows, words);
   }
   MVIT_CHECK_LAUNCH("gather_rows");
   return MVIT_OK;
@@ -531,6 +596,40 @@ int mvit_cast2d(const void* src, int64_t src_ld, int src_dtype, void* dst, int64
   else
     return mvit_set_error(MVIT_ERR_UNSUPPORTED, "cast2d: dtypes %d -> %d", src_dtype, dst_dtype);
   MVIT_CHECK_LAUNCH("cast2d");
+  return MVIT_OK;
+}
+
+int mvit_image_token_ranks(const int64_t* input_ids, const int64_t* labels, int64_t n_tokens, int64_t image_token_id,
+                           int64_t ignore_label, int32_t* rank, int64_t* positions, int64_t* counts, mvit_stream_t stream) {
+  MVIT_REQUIRE(input_ids && rank && positions && counts, "image_token_ranks: null pointer");
+  MVIT_REQUIRE(n_tokens >= 0 && n_tokens <= 0x7fffffffLL, "image_token_ranks: n_tokens %lld out of range", (long long)n_tokens);
+  hipLaunchKernelGGL(image_token_ranks_kernel, dim3(1), 1024, 0, S_(stream), input_ids, labels, n_tokens, image_token_id, ignore_label,
+                     rank, positions, counts);
+  MVIT_CHECK_LAUNCH("image_token_ranks");
+  return MVIT_OK;
+}
+
+int mvit_merge_rows(const void* embeds, const void* vision, const int32_t* rank, void* merged, int64_t n_tokens, int64_t n_vision,
+                    int64_t row_bytes, mvit_stream_t stream) {
+  MVIT_REQUIRE(embeds && rank && merged, "merge_rows: null pointer");
+  MVIT_REQUIRE(n_tokens >= 0 && n_vision >= 0 && row_bytes > 0 && row_bytes % 2 == 0, "merge_rows: bad sizes (row_bytes %lld)", (long long)row_bytes);
+  if (n_tokens == 0) return MVIT_OK;
+  const unsigned gy = (unsigned)clamp_grid(n_tokens, 65535);
+  const bool al = mvit_aligned16(embeds) && mvit_aligned16(merged) && (vision == nullptr || mvit_aligned16(vision));
+  if (row_bytes % 16 == 0 && al) {
+    const int64_t words = row_bytes / 16;
+    dim3 grid((unsigned)clamp_grid((words + 255) / 256, 64), gy);
+    hipLaunchKernelGGL((merge_rows_kernel<u32x4>), grid, 256, 0, S_(stream), (const u32x4*)embeds, (const u32x4*)vision, rank, (u32x4*)merged, n_tokens, n_vision, words);
+  } else if (row_bytes % 4 == 0) {
+    const int64_t words = row_bytes / 4;
+    dim3 grid((unsigned)clamp_grid((words + 255) / 256, 64), gy);
+    hipLaunchKernelGGL((merge_rows_kernel<uint32_t>), grid, 256, 0, S_(stream), (const uint32_t*)embeds, (const uint32_t*)vision, rank, (uint32_t*)merged, n_tokens, n_vision, words);
+  } else {
+    const int64_t words = row_bytes / 2;
+    dim3 grid((unsigned)clamp_grid((words + 255) / 256, 64), gy);
+    hipLaunchKernelGGL((merge_rows_kernel<uint16_t>), grid, 256, 0, S_(stream), (const uint16_t*)embeds, (const uint16_t*)vision, rank, (uint16_t*)merged, n_tokens, n_vision, words);
+  }
+  MVIT_CHECK_LAUNCH("merge_rows");
   return MVIT_OK;
 }
 

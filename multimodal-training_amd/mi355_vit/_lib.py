@@ -61,6 +61,8 @@ PROTOTYPES = {
     "mvit_cast2d": [_vp, _i64, _i32, _vp, _i64, _i32, _i64, _i64, _vp],
     "mvit_gemm": [C.POINTER(GemmArgs), _vp],
     "mvit_attn_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i64, _i32, _i32, _i64, _i64, _i64, _i64, _f32, _i32, _vp],
+    "mvit_image_token_ranks": [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp],
+    "mvit_merge_rows": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "mvit_adam_step": [_vp, _i32, _i64, C.c_double, C.c_double, C.c_double, C.c_double, _i32, _i32, _vp],
     "mvit_grad_sumsq": [_vp, _i32, _i64, _vp, _vp, _i32, _vp],
     "mvit_attn_bwd": [_vp] * 12 + [_i32, _i32, _i64, _i32, _i32] + [_i64] * 8 + [_f32, _i32, _vp],
