@@ -254,8 +254,8 @@ def cpu_baseline(cfg_kw, grid, seed, dtype, budget_s: float = 25.0):
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-trace", action="store_true", help="skip the per-kernel event pass (for profiler runs)")
@@ -326,7 +326,11 @@ def main() -> None:
         dom = max(mfma_tags, key=lambda k: mfma_tags[k]["ms"])
         d = mfma_tags[dom]
         ach = d["flops"] / (d["ms"] * 1e-3) / 1e12
-        roofline = {"bound": "mfma", "kernel": KERNEL_NAMES.get(dom, dom), "launches_per_step": d["launches"],
+        if dtype == torch.bfloat16:
+            kernel_name = KERNEL_NAMES.get(dom, dom)
+        else:  # the fp32 parity kernels: register-staged GEMM on v_mfma_f32_32x32x2_f32, one-lane-per-row attention
+            kernel_name = f"gemm_kernel<float, float, ...> ({dom})" if dom.startswith("gemm") else f"attn_*_f32 ({dom})"
+        roofline = {"bound": "mfma", "kernel": kernel_name, "launches_per_step": d["launches"],
                     "avg_launch_ms": d["ms"] / d["launches"], "achieved": ach, "peak": peak, "unit": "TFLOP/s",
                     "frac": ach / peak, "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, dom))}
         a_ms = sum(v["ms"] for t, v in summ.items() if t.startswith("attn"))
