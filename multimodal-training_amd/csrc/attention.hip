@@ -856,7 +856,7 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams
 }
 
 // ================================================================================================
-// Whole backward of a short segment (<= 64 rows, the windowed layers) in one wave: Q, K, V and dO of one
+// Whole backward of a short segment (<= 64 rows, the windowed layers) in one work-group: Q, K, V and dO of one
 // (segment, head) are staged in LDS once.  Pass A works in the dQ orientation (a lane owns a query), where
 // delta_q = sum_k P[q,k] * dP[q,k] (equal to dO_q . O_q, so O is never read) is a lane-local sum, and writes dQ;
 // pass B repeats the dK/dV kernel's tile loop on the staged tiles.  HBM traffic: four tiles in, three out.
@@ -1267,7 +1267,7 @@ int launch_fwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
 }
 template <int ND>
 int launch_bwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t s) {
-  // short segments (windows): one wave owns a whole 64-row block; long ones: 8 waves x 32 rows (2 waves per SIMD)
+  // short segments (windows): one work-group does the whole backward of a (segment, head); long ones: 8 waves x 32 rows
   if (max_seqlen <= 64) {
     dim3 grid(1, (unsigned)n_seg, (unsigned)p.nheads);
     if constexpr (ND <= 5) {
@@ -1368,7 +1368,7 @@ int mvit_attn_bwd(const void* q, const void* k, const void* v, const void* o, co
   const int vecw = dtype == MVIT_BF16 ? 8 : 4;
   const size_t part_bytes = (size_t)16 * nheads * (head_dim / vecw) * sizeof(float);
   if (dtype == MVIT_BF16 && max_seqlen <= 64 && head_dim <= 80) {
-    // the single-wave window kernel derives delta from P and dP
+    // the window kernel derives delta from P and dP itself
   } else if (head_dim % vecw == 0 && o_stride % vecw == 0 && do_stride % vecw == 0 && part_bytes <= 48 * 1024 && mvit_aligned16(o) && mvit_aligned16(d_o)) {
     const int dgrid = (int)((total + 15) / 16);
     if (dtype == MVIT_BF16)

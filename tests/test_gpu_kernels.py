@@ -376,7 +376,7 @@ def _attn_case(dtype, seglens, H, d, seed=0, qkv_packed=True):
     [
         ([64] * 6, 16, 80),  # windows
         ([64, 16, 48, 64, 32, 4], 4, 80),  # ragged edge windows
-        ([1, 17, 63, 33, 5], 2, 80),  # short windows of odd lengths (single-wave backward)
+        ([1, 17, 63, 33, 5], 2, 80),  # short windows of odd lengths (fused window backward)
         ([64, 20, 40], 2, 64),
         ([40, 64, 7], 2, 32),
         ([256, 256], 16, 80),  # cfg-1 full layer
