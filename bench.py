@@ -102,10 +102,10 @@ KERNEL_NAMES = {
     "gemm_nn_epi2": "gemm_dl_kernel<TO, TA=false, TB=false, EPI=BIAS_RES>",
     "gemm_nn_epi3": "gemm_dl_kernel<TO, TA=false, TB=false, EPI=BIAS_GELU>",
     "gemm_nn_epi4": "gemm_dl_kernel<TO, TA=false, TB=false, EPI=SWIGLU>",
-    "gemm_nt_epi0": "gemm_dl_kernel<TO, TA=false, TB=true, EPI=NONE>",
+    "gemm_nt_epi0": "gemm_dl_kernel<TO, TA=false, TB=true, EPI=NONE, MI16>",
     "gemm_nt_epi5": "gemm_dl_kernel<TO, TA=false, TB=true, EPI=SWIGLU_BWD>",
     "gemm_nt_epi6": "gemm_dl_kernel<TO, TA=false, TB=true, EPI=GELU_BWD>",
-    "gemm_tt_epi0": "gemm_dl_kernel<TO, TA=true, TB=true, EPI=NONE> + splitk_reduce_kernel",
+    "gemm_tt_epi0": "gemm_dl_kernel<TO, TA=true, TB=true, EPI=NONE, MI16> + splitk_reduce_kernel",
     "attn_fwd_full": "attn_fwd_mfma<5, 8, 32, true, 2, 4>",
     "attn_bwd_full": "attn_delta_kernel + attn_bwd_dkdv_mfma<5, 8, 2> + attn_bwd_dq_mfma<5, 8, 2>",
     "attn_fwd_window": "attn_fwd_mfma<5, 2, 64, false, 2, 4>",

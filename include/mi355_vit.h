@@ -134,7 +134,8 @@ typedef struct mvit_gemm_args {
   int trans_a;   /* 0: A is [M,K] (lda >= K);  1: A is [K,M] (lda >= M) */
   int trans_b;   /* 0: B is [N,K] (ldb >= K);  1: B is [K,N] (ldb >= N) */
   int epilogue;  /* MVIT_EPI_* */
-  int reserved;  /* main-loop variant: 0 = default; 1 = register-staged, 3 = direct-to-LDS (tuning / tests) */
+  int reserved;  /* main-loop variant: 0 = default; 1 = register-staged, 3 = direct-to-LDS with the MFMA shape chosen per
+                    operand layout, 5 / 7 = direct-to-LDS on 16x16x32 / 32x32x16 MFMA only (tuning / tests) */
   int64_t M, N, K;
   const void* A;
   int64_t lda;

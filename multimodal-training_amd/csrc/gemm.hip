@@ -425,14 +425,15 @@ struct EpiPre {
 // Epilogue shared by every main loop.  acc[a][b][4*j+i] is C[m0 + wm*WM + a*32 + 8*j + 4*(l/32) + i][wave column
 // b*32 + l%32].  Pass a: every wave parks its a-th 32-row sub-tile in LDS (fp32, [(BM/WM)*32 rows][BN + 8]), then
 // the block walks the pass in 8-column groups.  The caller guarantees that no wave still reads operands from LDS.
-template <typename T, typename TO, int EPI, int BM, int BN, int WM, int WN, int NTHREADS>
+template <typename T, typename TO, int EPI, int BM, int BN, int WM, int WN, int NTHREADS, bool MI16 = false>
 __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[WM / 32][WN / 32], unsigned char* smem_raw,
                                              int64_t m0, int64_t n0, int wm, int wn, int slice,
                                              EpiPre<T, EPI, BM, BN, WM, NTHREADS>& ep) {
   constexpr int MT = WM / 32, NT = WN / 32;
   constexpr bool DUAL = (EPI == MVIT_EPI_SWIGLU);
   const int l = threadIdx.x & 63;
-  constexpr int SP = BN + 8;
+  // MI16: acc[a][b] holds the four 16x16 results of the 32x32 block, [(ra*2 + cb)*4 + i] = C[16*ra + 4*(l/16) + i][16*cb + l%16]
+  constexpr int SP = MI16 ? BN + 4 : BN + 8;  // staging pitch (floats): keeps the parking stores of either layout off each other's banks
   constexpr int PASS_ROWS = (BM / WM) * 32;
   constexpr int NCOLS = DUAL ? BN / 2 : BN;
   constexpr int GROUPS = NCOLS / 8;
@@ -490,10 +491,18 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
           int col;
           if (DUAL) col = (b / (NT / 2)) * (BN / 2) + wn * (WN / 2) + (b % (NT / 2)) * 32 + lc;
           else col = wn * WN + b * 32 + lc;
+          if constexpr (MI16) {
 #pragma unroll
-          for (int j = 0; j < 4; ++j)
+            for (int q = 0; q < 4; ++q)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) stage[(wm * 32 + 8 * j + lr + i) * SP + col] = acc[a][b][4 * j + i];
+              for (int i = 0; i < 4; ++i)
+                stage[(wm * 32 + 16 * (q >> 1) + 4 * (l >> 4) + i) * SP + (col - lc) + 16 * (q & 1) + (l & 15)] = acc[a][b][4 * q + i];
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) stage[(wm * 32 + 8 * j + lr + i) * SP + col] = acc[a][b][4 * j + i];
+          }
         }
         __syncthreads();
 #pragma unroll
@@ -535,10 +544,18 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
       int col;
       if (DUAL) col = (b / (NT / 2)) * (BN / 2) + wn * (WN / 2) + (b % (NT / 2)) * 32 + lc;
       else col = wn * WN + b * 32 + lc;
+      if constexpr (MI16) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+        for (int q = 0; q < 4; ++q)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) stage[(wm * 32 + 8 * j + lr + i) * SP + col] = acc[a][b][4 * j + i];
+          for (int i = 0; i < 4; ++i)
+            stage[(wm * 32 + 16 * (q >> 1) + 4 * (l >> 4) + i) * SP + (col - lc) + 16 * (q & 1) + (l & 15)] = acc[a][b][4 * q + i];
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) stage[(wm * 32 + 8 * j + lr + i) * SP + col] = acc[a][b][4 * j + i];
+      }
     }
     __syncthreads();
     for (int c = threadIdx.x; c < PASS_ROWS * GROUPS; c += NTHREADS) {
@@ -718,7 +735,7 @@ __device__ __forceinline__ void wait_vm() {
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-template <bool TR, bool DUAL, int NW>
+template <bool TR, bool DUAL, int NW, bool MI16 = false>
 struct DlOperand {
   static constexpr int CPT = DL<NW>::CPT, WN = DL<NW>::WN;
   unsigned voff[CPT];  // byte offset of this lane's 16-byte chunks from `base`
@@ -744,7 +761,9 @@ struct DlOperand {
         voff[i] = (unsigned)(((grow - row0) * ld + c * 8) * 2);
       } else {
         const int kr = 2 * q + (l >> 5);
-        int ch = (l & 31) ^ ((kr & 3) << 2);
+        // MI16: the four 16-lane groups of a transposing read sit 8 k-rows apart; odd multiples of 8 are moved
+        // by two chunks so that two neighbouring groups never share banks
+        int ch = (l & 31) ^ ((kr & 3) << 2) ^ (MI16 ? ((kr >> 3) & 1) << 1 : 0);
         if (row0 + ch * 8 >= limit) ch = 0;
         voff[i] = (unsigned)((kr * ld + ch * 8) * 2);
       }
@@ -779,11 +798,26 @@ struct DlOperand {
 };
 
 // MFMA operand fetch for the DL layout: sub-tile `a` (32 rows) of the wave, 16-wide contraction step ks, stage s.
-template <bool TR, int NSUB>
+template <bool TR, int NSUB, bool MI16 = false>
 struct DlFrag {
-  unsigned off[TR ? NSUB : 2];
+  unsigned off[MI16 ? (TR ? 2 * NSUB : 1) : (TR ? NSUB : 2)];
   __device__ __forceinline__ void init(int rowbase, unsigned region) {
     const int l = threadIdx.x & 63;
+    if constexpr (MI16) {
+      // v_mfma_f32_16x16x32 operand: lane l holds row l%16 of a 16-row block, contraction 8*(l/16) .. +7 of the 32-wide stage
+      if (!TR) {
+        const int r = rowbase + (l & 15);  // blocks are 16 rows apart: (r >> 2) & 3 is the same for every block
+        off[0] = region + r * 64 + (((l >> 4) ^ ((r >> 2) & 3)) << 4);
+      } else {
+        const int G = l >> 4, i = l & 15, k = 8 * G + (i >> 2);
+#pragma unroll
+        for (int a = 0; a < 2 * NSUB; ++a) {
+          const int ch = (rowbase + a * 16) / 8 + ((i & 3) >> 1);
+          off[a] = region + k * 512 + ((ch ^ ((k & 3) << 2) ^ (((k >> 3) & 1) << 1)) << 4) + (i & 1) * 8;
+        }
+      }
+      return;
+    }
     if (!TR) {
       const int x = ((l & 31) >> 2) & 3;
 #pragma unroll
@@ -797,6 +831,20 @@ struct DlFrag {
         const int ch = (rowbase + a * 32) / 8 + 2 * (G & 1) + ((i & 3) >> 1);
         off[a] = region + (8 * (G >> 1) + (i >> 2)) * 512 + ((ch ^ (((i >> 2) & 3) << 2)) << 4) + (i & 1) * 8;
       }
+    }
+  }
+  // MI16: fragment of the 16-row block `blk` of the wave for the whole 32-wide stage s
+  __device__ __forceinline__ bf16x8 read16(const unsigned char* smem, int blk, int s) const {
+    if (!TR) {
+      return *reinterpret_cast<const bf16x8*>(smem + off[0] + blk * 16 * 64 + s * DL_TILE_BYTES);
+    } else {
+      typedef s16x4 __attribute__((address_space(3))) * lds_ptr_t;
+      const unsigned char* p = smem + off[blk] + s * DL_TILE_BYTES;
+      s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(p));
+      s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(p + 4 * 512));
+      typedef short s16x8 __attribute__((ext_vector_type(8)));
+      s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      return __builtin_bit_cast(bf16x8, both);
     }
   }
   __device__ __forceinline__ bf16x8 read(const unsigned char* smem, int a, int ks, int s) const {
@@ -823,7 +871,7 @@ __device__ __forceinline__ void wait_tiles(int n) {
   else wait_vm<0>();
 }
 
-template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, int NW>
+template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, int NW, bool MI16 = false>
 __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmParams p) {
   using T = bf16_t;
   using D = DL<NW>;
@@ -837,8 +885,8 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
   const int per_xcd = (total + 7) / 8;
   const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wv / WGN, wn = wv % WGN;
-  DlFrag<TA, MT> ra;
-  DlFrag<TB, NT> rb;
+  DlFrag<TA, MT, MI16> ra;
+  DlFrag<TB, NT, MI16> rb;
   ra.init(wm * WM, 0);
   rb.init(wn * WN, NSTAGE * TILE);
   typedef __attribute__((address_space(3))) unsigned char lds_byte;
@@ -867,8 +915,8 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
 
   EpiPre<T, EPI, BM, BN, WM, D::NTHREADS> ep;
   ep.init(p, m0, n0);
-  DlOperand<TA, false, NW> la;
-  DlOperand<TB, DUAL, NW> lb;
+  DlOperand<TA, false, NW, MI16> la;
+  DlOperand<TB, DUAL, NW, MI16> lb;
   la.init(static_cast<const T*>(p.A), nullptr, p.lda, m0, p.M, k_begin, wv);
   lb.init(static_cast<const T*>(p.B), static_cast<const T*>(p.B2), p.ldb, n0, p.N, k_begin, wv);
   const int klen = (int)(k_end - k_begin);
@@ -886,7 +934,7 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
 #pragma unroll
   for (int t = 0; t < NSTAGE - 1; ++t) issue(t, t);
 
-  bf16x8 fa[2][MT], fb[2][NT];
+  [[maybe_unused]] bf16x8 fa[2][MT], fb[2][NT];
   for (int t0 = 0; t0 < T_; t0 += NSTAGE) {
 #pragma unroll
     for (int s = 0; s < NSTAGE; ++s) {
@@ -899,6 +947,29 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
       __builtin_amdgcn_s_barrier();  // every wave's share of that tile is in LDS; stage (s-1) has been consumed
       issue(t + NSTAGE - 1, (s + NSTAGE - 1) % NSTAGE);
 
+      if constexpr (MI16) {
+        // one 32-wide step per stage on v_mfma_f32_16x16x32_bf16: 2*MT x 2*NT blocks of 16x16
+        bf16x8 ga[2 * MT], gb[2 * NT];
+#pragma unroll
+        for (int a = 0; a < 2 * MT; ++a) ga[a] = ra.read16(smem_raw, a, s);
+#pragma unroll
+        for (int b = 0; b < 2 * NT; ++b) gb[b] = rb.read16(smem_raw, b, s);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int a = 0; a < 2 * MT; ++a)
+#pragma unroll
+          for (int b = 0; b < 2 * NT; ++b) {
+            f32x16& blk = acc[a >> 1][b >> 1];
+            const int q = (a & 1) * 2 + (b & 1);
+            f32x4 c = {blk[4 * q], blk[4 * q + 1], blk[4 * q + 2], blk[4 * q + 3]};
+            c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[a], gb[b], c, 0, 0, 0);
+            blk[4 * q] = c[0];
+            blk[4 * q + 1] = c[1];
+            blk[4 * q + 2] = c[2];
+            blk[4 * q + 3] = c[3];
+          }
+        __builtin_amdgcn_sched_barrier(0);
+      } else {
 #pragma unroll
       for (int a = 0; a < MT; ++a) fa[0][a] = ra.read(smem_raw, a, 0, s);
 #pragma unroll
@@ -921,10 +992,11 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
         for (int b = 0; b < NT; ++b)
           acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][a], fb[1][b], acc[a][b], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
+      }
     }
   }
   __syncthreads();  // operands fully consumed before LDS is reused by the epilogue
-  run_epilogue<T, TO, EPI, BM, BN, WM, WN, D::NTHREADS>(p, acc, smem_raw, m0, n0, wm, wn, slice, ep);
+  run_epilogue<T, TO, EPI, BM, BN, WM, WN, D::NTHREADS, MI16>(p, acc, smem_raw, m0, n0, wm, wn, slice, ep);
   __syncthreads();  // the staging area is free again before the next tile's operands land in it
   }
 }
@@ -971,13 +1043,13 @@ int launch(const GemmParams& p, hipStream_t stream) {
   return MVIT_OK;
 }
 
-template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, int NW>
+template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, int NW, bool MI16 = false>
 int launch_dl(const GemmParams& p, hipStream_t stream) {
   using D = DL<NW>;
   const size_t operands = 2 * (size_t)NSTAGE * D::TILE_BYTES;
   const size_t staging = (size_t)(D::BM / D::WM) * 32 * (D::BN + 8) * sizeof(float);
   const size_t lds = operands > staging ? operands : staging;
-  auto kern = gemm_dl_kernel<TO, TA, TB, EPI, NSTAGE, NW>;
+  auto kern = gemm_dl_kernel<TO, TA, TB, EPI, NSTAGE, NW, MI16>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -1008,7 +1080,12 @@ int launch_dl(const GemmParams& p, hipStream_t stream) {
 template <typename T, typename TO, bool TA, bool TB, int EPI>
 int launch_var(int var, const GemmParams& p, hipStream_t s) {
   if constexpr (sizeof(T) == 2) {
-    if (var == 3) return launch_dl<TO, TA, TB, EPI, 4, 8>(p, s);
+    // default: v_mfma_f32_16x16x32_bf16 for the plain GEMMs with an operand behind the transposing LDS read
+    // (weight gradients +6 %, input gradients +1 % on real data), v_mfma_f32_32x32x16_bf16 for the forward GEMMs
+    // (both operands row-major: 3-5 % faster that way) and for the fused backward epilogues; 5 / 7 force one shape
+    if (var == 3) return (TB && EPI == MVIT_EPI_NONE) ? launch_dl<TO, TA, TB, EPI, 4, 8, true>(p, s) : launch_dl<TO, TA, TB, EPI, 4, 8>(p, s);
+    if (var == 5) return launch_dl<TO, TA, TB, EPI, 4, 8, true>(p, s);
+    if (var == 7) return launch_dl<TO, TA, TB, EPI, 4, 8>(p, s);
 
   }
   if (var == 1 || var >= 3) return launch<T, TO, TA, TB, EPI, 1>(p, s);
@@ -1086,7 +1163,7 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
   const size_t es = a->dtype == MVIT_BF16 ? 2 : 4, eo = a->out_dtype == MVIT_BF16 ? 2 : 4;
   p.vec_ok = vec16(a->C, a->ldc, eo) && vec16(a->R, a->ldr, es) && vec16(a->aux, a->ldaux, es) && vec16(a->bias, 0, es) &&
              vec16(a->bias2, 0, es) && (a->aux_off * (int64_t)(es < eo ? es : eo)) % 16 == 0;
-  int var = (a->reserved == 1 || a->reserved == 3) ? a->reserved : 3;  // 0 (or anything else) = default
+  int var = (a->reserved == 1 || a->reserved == 3 || a->reserved == 5 || a->reserved == 7) ? a->reserved : 3;  // 0 (or anything else) = default
   if (var >= 3 && (a->lda > (1ll << 22) || a->ldb > (1ll << 22))) var = 1;  // 32-bit lane offsets  // tile / wave layout, see Waves<>
   const int BM = 256, BN = 256;
   const int n_per_block = (epi == MVIT_EPI_SWIGLU) ? BN / 2 : BN;

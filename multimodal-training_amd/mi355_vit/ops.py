@@ -17,7 +17,7 @@ _DT = {torch.float32: F32, torch.bfloat16: BF16}
 N_PARTIAL = 1024  # work-groups (= partial rows) of the RMSNorm backward: 4 per CU keep enough loads in flight
 
 GEMM_PANEL = int(_os.environ.get("MI355_VIT_GEMM_PANEL", "0"))  # bits 0-7: tile-order panel width override (0: library default); bits 8-15: tuning switches
-GEMM_VARIANT = int(_os.environ.get("MI355_VIT_GEMM_VARIANT", "0"))  # GEMM main loop: 0 default, 1 register-staged, 3 direct-to-LDS
+GEMM_VARIANT = int(_os.environ.get("MI355_VIT_GEMM_VARIANT", "0"))  # GEMM main loop: 0 default, 1 register-staged, 3 direct-to-LDS, 5 / 7 one MFMA shape only
 
 _trace = None  # optional list collecting (tag, info, start_event, end_event) per tagged launch
 
