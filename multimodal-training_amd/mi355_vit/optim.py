@@ -135,7 +135,10 @@ class FusedAdam(torch.optim.Adam):
         # which parameters take part (those with a gradient) and where they and their moments live rarely changes:
         # the table is rebuilt only when it does; per step only gradient addresses and scalars are refreshed
         key = tuple((id(p), p.data_ptr()) for group in self.param_groups for p in group["params"] if p.grad is not None)
-        if key != self._plan_key:
+        stale = key != self._plan_key or any(
+            int(bk.step_tensors[0].item()) != int(bk.steps[0]) or int(bk.step_tensors[-1].item()) != int(bk.steps[-1])
+            for bk in self._plan)  # step counters edited from outside (cheap spot check of the host mirror)
+        if stale:
             self._plan = self._make_plan()
             self._plan_key = key
         lib = _lib.load()
