@@ -433,7 +433,11 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
   constexpr bool DUAL = (EPI == MVIT_EPI_SWIGLU);
   const int l = threadIdx.x & 63;
   // MI16: acc[a][b] holds the four 16x16 results of the 32x32 block, [(ra*2 + cb)*4 + i] = C[16*ra + 4*(l/16) + i][16*cb + l%16]
-  constexpr int SP = MI16 ? BN + 4 : BN + 8;  // staging pitch (floats): keeps the parking stores of either layout off each other's banks
+  // Staging rows are BN floats with no padding; 16-column chunks of a row are permuted by the row instead, so that the
+  // rows one parking store touches (4 apart: four of them with the 16x16 results, two with the 32x32 ones) fall on
+  // different banks.  Groups of 8 columns stay contiguous for the read-out.
+  constexpr int SP = BN;
+  auto swz = [](int row) { return MI16 ? ((row >> 2) & 3) << 4 : ((row >> 2) & 1) << 5; };
   constexpr int PASS_ROWS = (BM / WM) * 32;
   constexpr int NCOLS = DUAL ? BN / 2 : BN;
   constexpr int GROUPS = NCOLS / 8;
@@ -496,12 +500,12 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
             for (int q = 0; q < 4; ++q)
 #pragma unroll
               for (int i = 0; i < 4; ++i)
-                stage[(wm * 32 + 16 * (q >> 1) + 4 * (l >> 4) + i) * SP + (col - lc) + 16 * (q & 1) + (l & 15)] = acc[a][b][4 * q + i];
+                stage[(wm * 32 + 16 * (q >> 1) + 4 * (l >> 4) + i) * SP + (((col - lc) + 16 * (q & 1) + (l & 15)) ^ swz(4 * (l >> 4)))] = acc[a][b][4 * q + i];
           } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
-              for (int i = 0; i < 4; ++i) stage[(wm * 32 + 8 * j + lr + i) * SP + col] = acc[a][b][4 * j + i];
+              for (int i = 0; i < 4; ++i) stage[(wm * 32 + 8 * j + lr + i) * SP + (col ^ swz(lr))] = acc[a][b][4 * j + i];
           }
         }
         __syncthreads();
@@ -509,7 +513,7 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
         for (int it = 0; it < ITEMS; ++it) {
           const int c = threadIdx.x + NTHREADS * it, row = c / GROUPS, cg = c % GROUPS;
           const int64_t m = m0 + (row / 32) * WM + a * 32 + (row % 32), n = n0 + cg * 8;
-          const float* sp = stage + row * SP + cg * 8;
+          const float* sp = stage + row * SP + ((cg * 8) ^ swz(row));
           const f32x4 v0 = *reinterpret_cast<const f32x4*>(sp), v1 = *reinterpret_cast<const f32x4*>(sp + 4);
           float v[8] = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
           float u[8];
@@ -549,12 +553,12 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
         for (int q = 0; q < 4; ++q)
 #pragma unroll
           for (int i = 0; i < 4; ++i)
-            stage[(wm * 32 + 16 * (q >> 1) + 4 * (l >> 4) + i) * SP + (col - lc) + 16 * (q & 1) + (l & 15)] = acc[a][b][4 * q + i];
+            stage[(wm * 32 + 16 * (q >> 1) + 4 * (l >> 4) + i) * SP + (((col - lc) + 16 * (q & 1) + (l & 15)) ^ swz(4 * (l >> 4)))] = acc[a][b][4 * q + i];
       } else {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) stage[(wm * 32 + 8 * j + lr + i) * SP + col] = acc[a][b][4 * j + i];
+          for (int i = 0; i < 4; ++i) stage[(wm * 32 + 8 * j + lr + i) * SP + (col ^ swz(lr))] = acc[a][b][4 * j + i];
       }
     }
     __syncthreads();
@@ -564,7 +568,7 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
       const int64_t n = n0 + cg * 8;
       if (m >= p.M || n >= p.N) continue;
       float v[8], u[8];
-      const float* sp = stage + row * SP + cg * 8;
+      const float* sp = stage + row * SP + ((cg * 8) ^ swz(row));
       const f32x4 v0 = *reinterpret_cast<const f32x4*>(sp), v1 = *reinterpret_cast<const f32x4*>(sp + 4);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -862,6 +866,13 @@ struct DlFrag {
   }
 };
 
+// Whether gemm_dl_kernel starts the next tile's loads before the epilogue of the current one: the weight-gradient
+// GEMMs (A transposed) with a plain or bias epilogue.  Measured on the full tower: those kernels get 2-3 % faster and
+// the step follows; the forward and input-gradient GEMMs also get 1-3 % faster alone, but the step with the
+// weight gradients running beside them on a second stream gets slower, so they keep starting a tile after the
+// epilogue.  The fused epilogues have no registers to spare for the next tile's addresses.
+constexpr bool dl_prefetches(int epi, bool ta) { return (epi == MVIT_EPI_NONE || epi == MVIT_EPI_BIAS) && ta; }
+
 // Wait until at most n K tiles' loads (PER per lane each) are still in flight.
 template <int PER>
 __device__ __forceinline__ void wait_tiles(int n) {
@@ -894,16 +905,59 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
 
   // Persistent work-groups: the grid has at most one work-group per CU; work-group (xcd, slot) walks that XCD's
   // tile range with stride slots-per-XCD, the order a one-tile-per-work-group grid would be dispatched in.
-  for (int idx = blockIdx.x >> 3; idx < per_xcd; idx += gridDim.x >> 3) {
-  const int work = (blockIdx.x & 7) * per_xcd + idx;
-  if (work >= total) break;
-  const int slice = work / tiles, tile = work % tiles;
-  int tm, tn;
-  tile_coords(p, tile, tm, tn);
-  const int64_t k_begin = (int64_t)slice * p.k_chunk;
-  const int64_t k_end = p.split_k > 1 ? (k_begin + p.k_chunk < p.K ? k_begin + p.k_chunk : p.K) : p.K;
+  // Where dl_prefetches() says so, the first two K tiles of a work-group's next output tile are requested before the
+  // epilogue of the current one, so they travel while the results are parked and stored: the epilogue then stages
+  // through the later B stages and the LDS behind them, which those loads do not touch.
+  constexpr bool PREFETCH = dl_prefetches(EPI, TA);
+  constexpr int EARLY = PREFETCH ? (NSTAGE - 1 < 2 ? NSTAGE - 1 : 2) : NSTAGE - 1;  // K tiles requested by start_tile
+  constexpr int STAGING_OFF = PREFETCH ? (NSTAGE + EARLY) * TILE : 0;
+  DlOperand<TA, false, NW, MI16> la;
+  DlOperand<TB, DUAL, NW, MI16> lb;
+  int T_ = 0, k_tail = 0;  // of the tile whose operands are being loaded
+  auto issue = [&](int t, int s) {  // K tile t into stage s (both wave-uniform)
+    if (t >= T_) return;
+    if (k_tail != 0 && t == T_ - 1) {
+      la.issue_tail(smem_raw + s * TILE + wv * SLICE, k_tail, wv);
+      lb.issue_tail(smem_raw + (NSTAGE + s) * TILE + wv * SLICE, k_tail, wv);
+    } else {
+      la.issue(lds0 + s * TILE);
+      lb.issue(lds0 + (NSTAGE + s) * TILE);
+    }
+  };
   constexpr int N_PER_BLOCK = DUAL ? BN / 2 : BN;
-  const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * N_PER_BLOCK;
+  int next_slice = 0;
+  int64_t next_m0 = 0, next_n0 = 0;
+  // decodes work item `idx` of this work-group's XCD and starts its first loads; false past the end
+  auto start_tile = [&](int idx) -> bool {
+    if (idx >= per_xcd) return false;
+    const int work = (blockIdx.x & 7) * per_xcd + idx;
+    if (work >= total) return false;
+    next_slice = work / tiles;
+    int tm, tn;
+    tile_coords(p, work % tiles, tm, tn);
+    const int64_t k_begin = (int64_t)next_slice * p.k_chunk;
+    const int64_t k_end = p.split_k > 1 ? (k_begin + p.k_chunk < p.K ? k_begin + p.k_chunk : p.K) : p.K;
+    next_m0 = (int64_t)tm * BM;
+    next_n0 = (int64_t)tn * N_PER_BLOCK;
+    la.init(static_cast<const T*>(p.A), nullptr, p.lda, next_m0, p.M, k_begin, wv);
+    lb.init(static_cast<const T*>(p.B), static_cast<const T*>(p.B2), p.ldb, next_n0, p.N, k_begin, wv);
+    const int klen = (int)(k_end - k_begin);
+    T_ = (klen + DL_BK - 1) / DL_BK;
+    k_tail = klen % DL_BK;
+#pragma unroll
+    for (int t = 0; t < EARLY; ++t) issue(t, t);
+    return true;
+  };
+  int idx = blockIdx.x >> 3;
+  [[maybe_unused]] bool have = PREFETCH ? start_tile(idx) : true;
+  while (true) {
+  if constexpr (PREFETCH) {
+    if (!have) break;
+  } else {
+    if (!start_tile(idx)) break;
+  }
+  const int slice = next_slice;
+  const int64_t m0 = next_m0, n0 = next_n0;
 
   f32x16 acc[MT][NT];
 #pragma unroll
@@ -915,24 +969,8 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
 
   EpiPre<T, EPI, BM, BN, WM, D::NTHREADS> ep;
   ep.init(p, m0, n0);
-  DlOperand<TA, false, NW, MI16> la;
-  DlOperand<TB, DUAL, NW, MI16> lb;
-  la.init(static_cast<const T*>(p.A), nullptr, p.lda, m0, p.M, k_begin, wv);
-  lb.init(static_cast<const T*>(p.B), static_cast<const T*>(p.B2), p.ldb, n0, p.N, k_begin, wv);
-  const int klen = (int)(k_end - k_begin);
-  const int T_ = (klen + DL_BK - 1) / DL_BK, k_tail = klen % DL_BK;
-  auto issue = [&](int t, int s) {  // K tile t into stage s (both wave-uniform)
-    if (t >= T_) return;
-    if (k_tail != 0 && t == T_ - 1) {
-      la.issue_tail(smem_raw + s * TILE + wv * SLICE, k_tail, wv);
-      lb.issue_tail(smem_raw + (NSTAGE + s) * TILE + wv * SLICE, k_tail, wv);
-    } else {
-      la.issue(lds0 + s * TILE);
-      lb.issue(lds0 + (NSTAGE + s) * TILE);
-    }
-  };
 #pragma unroll
-  for (int t = 0; t < NSTAGE - 1; ++t) issue(t, t);
+  for (int t = EARLY; t < NSTAGE - 1; ++t) issue(t, t);  // the stages the previous tile's epilogue was using
 
   [[maybe_unused]] bf16x8 fa[2][MT], fb[2][NT];
   for (int t0 = 0; t0 < T_; t0 += NSTAGE) {
@@ -995,9 +1033,11 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
       }
     }
   }
-  __syncthreads();  // operands fully consumed before LDS is reused by the epilogue
-  run_epilogue<T, TO, EPI, BM, BN, WM, WN, D::NTHREADS, MI16>(p, acc, smem_raw, m0, n0, wm, wn, slice, ep);
-  __syncthreads();  // the staging area is free again before the next tile's operands land in it
+  __syncthreads();  // operands fully consumed before the next tile's first loads (or the epilogue) overwrite them
+  idx += gridDim.x >> 3;
+  if constexpr (PREFETCH) have = start_tile(idx);
+  run_epilogue<T, TO, EPI, BM, BN, WM, WN, D::NTHREADS, MI16>(p, acc, smem_raw + STAGING_OFF, m0, n0, wm, wn, slice, ep);
+  __syncthreads();  // the staging area is free again before operands land in it
   }
 }
 
@@ -1046,9 +1086,12 @@ int launch(const GemmParams& p, hipStream_t stream) {
 template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, int NW, bool MI16 = false>
 int launch_dl(const GemmParams& p, hipStream_t stream) {
   using D = DL<NW>;
-  const size_t operands = 2 * (size_t)NSTAGE * D::TILE_BYTES;
-  const size_t staging = (size_t)(D::BM / D::WM) * 32 * (D::BN + 8) * sizeof(float);
-  const size_t lds = operands > staging ? operands : staging;
+  constexpr size_t operands = 2 * (size_t)NSTAGE * D::TILE_BYTES;
+  constexpr size_t staging = (size_t)(D::BM / D::WM) * 32 * D::BN * sizeof(float);
+  // with prefetching the staging area starts behind the B stages that the next tile's first two K tiles arrive in
+  constexpr size_t staging_end = dl_prefetches(EPI, TA) ? (NSTAGE + (NSTAGE - 1 < 2 ? NSTAGE - 1 : 2)) * D::TILE_BYTES + staging : staging;
+  constexpr size_t lds = staging_end > operands ? staging_end : operands;
+  static_assert(lds <= 160 * 1024, "operand stages plus the epilogue staging area exceed the LDS of a CU");
   auto kern = gemm_dl_kernel<TO, TA, TB, EPI, NSTAGE, NW, MI16>;
   static bool attr_set = false;
   if (!attr_set) {
@@ -1083,9 +1126,10 @@ int launch_var(int var, const GemmParams& p, hipStream_t s) {
     // default: v_mfma_f32_16x16x32_bf16 for the plain GEMMs with an operand behind the transposing LDS read
     // (weight gradients +6 %, input gradients +1 % on real data), v_mfma_f32_32x32x16_bf16 for the forward GEMMs
     // (both operands row-major: 3-5 % faster that way) and for the fused backward epilogues; 5 / 7 force one shape
-    if (var == 3) return (TB && EPI == MVIT_EPI_NONE) ? launch_dl<TO, TA, TB, EPI, 4, 8, true>(p, s) : launch_dl<TO, TA, TB, EPI, 4, 8>(p, s);
-    if (var == 5) return launch_dl<TO, TA, TB, EPI, 4, 8, true>(p, s);
-    if (var == 7) return launch_dl<TO, TA, TB, EPI, 4, 8>(p, s);
+    constexpr int NS = 4;
+    if (var == 3) return (TB && EPI == MVIT_EPI_NONE) ? launch_dl<TO, TA, TB, EPI, NS, 8, true>(p, s) : launch_dl<TO, TA, TB, EPI, NS, 8>(p, s);
+    if (var == 5) return launch_dl<TO, TA, TB, EPI, NS, 8, true>(p, s);
+    if (var == 7) return launch_dl<TO, TA, TB, EPI, NS, 8>(p, s);
 
   }
   if (var == 1 || var >= 3) return launch<T, TO, TA, TB, EPI, 1>(p, s);
