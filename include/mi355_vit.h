@@ -250,6 +250,33 @@ int mvit_adam_step(const mvit_adam_tensor* tensors, int n_tensors, int64_t n_chu
 int mvit_grad_sumsq(const mvit_adam_tensor* tensors, int n_tensors, int64_t n_chunks, float* partial, double* out,
                     int dtype, mvit_stream_t stream);
 
+/* ---------------------------------------------------------------- input side: decoded frames -> pixel_values */
+
+#define MVIT_PIXEL_ROW 1176 /* 3 channels x 2 frames x 14 x 14: one row of pixel_values */
+
+/* One image or video of the batch: `frames` decoded RGB frames of height x width pixels, uint8, [frames][height]
+ * [width][3] contiguous in device memory, already resized (height and width multiples of 28).  first_row is the
+ * row of pixel_values its first patch goes to: the running sum of ceil(frames / 2) * (height / 14) * (width / 14).
+ * The table has n_images + 1 entries; the last one only carries first_row = total number of rows. */
+typedef struct mvit_image {
+  const uint8_t* pixels;
+  int32_t frames, height, width, reserved;
+  int64_t first_row;
+} mvit_image;
+
+/* pixel_values[first_row + r, :] for every image of the table, in one launch:
+ *   value = ((float)((double)byte * rescale) - mean[c]) / std[c]        (float32, then rounded to `dtype`)
+ * rows in the order (temporal pair, 2x2 merge block row, merge block column, row in block, column in block),
+ * columns in the order (channel, frame of the pair, y in patch, x in patch); a frame count that is odd is filled
+ * up by using the last frame twice (a still image fills both halves of its rows).  `images` is a device pointer,
+ * out is [total_rows, 1176] of dtype MVIT_F32 or MVIT_BF16.
+ * Replaces the rescale / normalise / patchify steps of the image processor that the reference runs on CPU
+ * workers through processor.apply_chat_template (python/data/preprocessing.py:134; transformers 4.57.0,
+ * Qwen2VLImageProcessor._preprocess) and the concatenation of python/data/collator.py:134-156; the cast to the
+ * model dtype is the one of the tower's first line (modeling_qwen2_5_vl.py, patch_embed input). */
+int mvit_patchify(const mvit_image* images, int n_images, int64_t total_rows, void* out, double rescale, float mean_r,
+                  float mean_g, float mean_b, float std_r, float std_g, float std_b, int dtype, mvit_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

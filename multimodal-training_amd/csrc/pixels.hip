@@ -1,0 +1,101 @@
+// Decoded RGB frames (uint8) -> rows of pixel_values for gfx950: rescale, normalise and cut into 14x14x2 patches in
+// the row order the vision tower expects, for a whole batch of images and videos in one launch.  HBM-bound: every
+// output row is 1176 values (4704 bytes in fp32) made from 2 x 588 input bytes; the input is read through the
+// caches byte by byte (a patch row is 42 contiguous bytes), the output leaves as 16-byte (fp32) or 8-byte (bf16)
+// stores, one wave per row and the four rows of a 2x2 merge block per work-group, so that a work-group reads one
+// 28x28 pixel square.
+//
+// The arithmetic is that of the image processor the reference calls (transformers 4.57.0,
+// Qwen2VLImageProcessor._preprocess: rescale in float64 rounded to float32, then (x - mean) / std in float32
+// with an IEEE division), so fp32 results can be compared bit for bit with a numpy restatement.
+#include "mvit_common.h"
+
+namespace {
+
+constexpr int PATCH = 14, TPS = 2, ROW = MVIT_PIXEL_ROW;
+constexpr int PLANE = PATCH * PATCH;   // 196 values of one (channel, frame) plane of a row
+constexpr int QUADS = PLANE / 4;       // 49 groups of four consecutive values per plane
+constexpr int ROW_QUADS = ROW / 4;     // 294
+
+struct Norm {
+  double rescale;
+  float mean[3], std[3];
+};
+
+__device__ __forceinline__ int find_image(const mvit_image* t, int n, int64_t row) {
+  int lo = 0, hi = n;  // invariant: t[lo].first_row <= row < t[hi].first_row
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (t[mid].first_row <= row) lo = mid;
+    else hi = mid;
+  }
+  return lo;
+}
+
+__device__ __forceinline__ void store4(float* dst, const float (&v)[4]) {
+  *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+}
+__device__ __forceinline__ void store4(bf16_t* dst, const float (&v)[4]) {
+  *reinterpret_cast<bf16x4*>(dst) = bf16x4{from_f32<bf16_t>(v[0]), from_f32<bf16_t>(v[1]), from_f32<bf16_t>(v[2]), from_f32<bf16_t>(v[3])};
+}
+
+template <typename TO>
+__global__ __launch_bounds__(256) void patchify_kernel(const mvit_image* __restrict__ images, int n_images, TO* __restrict__ out,
+                                                       int64_t total_rows, Norm nm) {
+#pragma clang fp contract(off)
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= total_rows) return;
+  const int lane = threadIdx.x & 63;
+  const mvit_image im = images[find_image(images, n_images, row)];
+  const int gh = im.height / PATCH, gw = im.width / PATCH;
+  if (im.frames <= 0 || gh <= 0 || gw <= 0 || ((gh | gw) & 1)) return;  // malformed entry: nothing is read
+  const int64_t local = row - im.first_row;
+  const int per_t = gh * gw;
+  const int t = (int)(local / per_t), rem = (int)(local % per_t);
+  // rem = ((block row * (gw / 2) + block column) * 2 + row in block) * 2 + column in block
+  const int blk = rem >> 2, hb = blk / (gw >> 1), wb = blk % (gw >> 1);
+  const int y0 = (hb * 2 + ((rem >> 1) & 1)) * PATCH, x0 = (wb * 2 + (rem & 1)) * PATCH;
+  if (t * TPS >= im.frames) return;  // first_row entries that promise more rows than the frames give
+  const int64_t line = (int64_t)im.width * 3, frame_bytes = line * im.height;
+  TO* dst = out + row * ROW;
+  for (int g = lane; g < ROW_QUADS; g += 64) {
+    const int c = g / (TPS * QUADS), tt = (g / QUADS) % TPS, q = g % QUADS;
+    int f = t * TPS + tt;
+    if (f >= im.frames) f = im.frames - 1;
+    const uint8_t* src = im.pixels + f * frame_bytes + y0 * line + x0 * 3 + c;
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int p = 4 * q + e, py = p / PATCH, px = p % PATCH;
+      const float x = (float)((double)src[py * line + px * 3] * nm.rescale);
+      v[e] = (x - nm.mean[c]) / nm.std[c];
+    }
+    store4(dst + 4 * g, v);
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int mvit_patchify(const mvit_image* images, int n_images, int64_t total_rows, void* out, double rescale, float mean_r,
+                  float mean_g, float mean_b, float std_r, float std_g, float std_b, int dtype, mvit_stream_t stream) {
+  MVIT_REQUIRE(images != nullptr && n_images > 0, "patchify: empty image table");
+  MVIT_REQUIRE(total_rows >= 0 && total_rows % 4 == 0 && total_rows / 4 <= 0x7fffffffLL,
+               "patchify: total_rows %lld must be a multiple of 4 (2x2 merge blocks) below 2^33", (long long)total_rows);
+  MVIT_REQUIRE(dtype == MVIT_BF16 || dtype == MVIT_F32, "patchify: dtype %d", dtype);
+  MVIT_REQUIRE(std_r != 0.f && std_g != 0.f && std_b != 0.f, "patchify: zero std");
+  if (total_rows == 0) return MVIT_OK;
+  MVIT_REQUIRE(out != nullptr && mvit_aligned16(out), "patchify: output must be a 16-byte aligned device pointer");
+  Norm nm{rescale, {mean_r, mean_g, mean_b}, {std_r, std_g, std_b}};
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const unsigned grid = (unsigned)(total_rows / 4);
+  if (dtype == MVIT_BF16)
+    hipLaunchKernelGGL((patchify_kernel<bf16_t>), dim3(grid), 256, 0, s, images, n_images, static_cast<bf16_t*>(out), total_rows, nm);
+  else
+    hipLaunchKernelGGL((patchify_kernel<float>), dim3(grid), 256, 0, s, images, n_images, static_cast<float*>(out), total_rows, nm);
+  MVIT_CHECK_LAUNCH("patchify");
+  return MVIT_OK;
+}
+
+}  // extern "C"

@@ -43,6 +43,15 @@ class AdamTensor(C.Structure):
 
 ADAM_CHUNK = 8192
 
+
+class Image(C.Structure):
+    """mvit_image: one image or video of the device-resident table of mvit_patchify."""
+
+    _fields_ = [("pixels", _vp), ("frames", _i32), ("height", _i32), ("width", _i32), ("reserved", _i32), ("first_row", _i64)]
+
+
+PIXEL_ROW = 1176
+
 # name -> argument types (every function returns int except the two noted below)
 PROTOTYPES = {
     "mvit_rot_pos_ids": [_vp, _i64, _i32, _vp],
@@ -65,6 +74,7 @@ PROTOTYPES = {
     "mvit_merge_rows": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "mvit_adam_step": [_vp, _i32, _i64, C.c_double, C.c_double, C.c_double, C.c_double, _i32, _i32, _vp],
     "mvit_grad_sumsq": [_vp, _i32, _i64, _vp, _vp, _i32, _vp],
+    "mvit_patchify": [_vp, _i32, _i64, _vp, C.c_double] + [_f32] * 6 + [_i32, _vp],
     "mvit_attn_bwd": [_vp] * 12 + [_i32, _i32, _i64, _i32, _i32] + [_i64] * 8 + [_f32, _i32, _vp],
 }
 EXPORTS = sorted(list(PROTOTYPES) + ["mvit_version", "mvit_last_error"])

@@ -1,0 +1,117 @@
+"""Parity of the input-side kernel (decoded frames -> pixel_values rows, through the C ABI) against the CPU oracle.
+
+float32 output is compared bit for bit (the oracle restates the image processor's arithmetic with its dtypes);
+bfloat16 output bit for bit against the oracle's float32 result rounded once, the cast the tower applies."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import pixels_oracle as po
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _announce(msg):
+    print(f"[case] {msg}", flush=True)
+
+
+def _batch(seed, shapes):
+    rng = np.random.default_rng(seed)
+    return [rng.integers(0, 256, size=(f, h, w, 3), dtype=np.uint8) for f, h, w in shapes]
+
+
+def _run(images, **kw):
+    from mi355_vit.pixels import patchify
+
+    out, grid = patchify([torch.from_numpy(im).to(DEV) for im in images], **kw)
+    torch.cuda.synchronize()
+    return out.cpu(), grid
+
+
+RAGGED = [(1, 56, 84), (1, 28, 28), (2, 84, 56), (3, 28, 112), (1, 364, 252), (5, 56, 56), (1, 112, 28)]
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_patchify_bit_exact_against_oracle_ragged_images_and_videos(seed):
+    _announce(f"patchify fp32 ragged seed={seed}")
+    images = _batch(seed, RAGGED)
+    got, grid = _run(images)
+    ref, ref_grid = po.patchify_batch(images)
+    assert grid.dtype == torch.int64 and not grid.is_cuda and grid.tolist() == ref_grid.tolist()
+    assert got.dtype == torch.float32 and tuple(got.shape) == ref.shape
+    assert np.array_equal(got.numpy().view(np.uint32), ref.view(np.uint32))
+
+
+def test_patchify_bf16_is_the_rounded_fp32_result():
+    _announce("patchify bf16")
+    images = _batch(2, RAGGED[:5])
+    got, _ = _run(images, dtype=torch.bfloat16)
+    ref = torch.from_numpy(po.patchify_batch(images)[0]).to(torch.bfloat16)
+    assert got.dtype == torch.bfloat16 and torch.equal(got, ref)
+
+
+def test_patchify_every_byte_value_other_constants_and_out_argument():
+    _announce("patchify all byte values, custom constants")
+    ramp = np.arange(28 * 28 * 3, dtype=np.int64).reshape(1, 28, 28, 3) % 256
+    images = [ramp.astype(np.uint8), _batch(3, [(2, 28, 56)])[0]]
+    mean, std, scale = (0.5, 0.25, 0.125), (0.5, 0.3, 0.7), 1.0 / 127.5
+    from mi355_vit.pixels import patchify
+
+    out = torch.full((4 + 8, 1176), float("nan"), device=DEV)
+    got, _ = patchify([torch.from_numpy(im).to(DEV) for im in images], image_mean=mean, image_std=std, rescale_factor=scale, out=out)
+    assert got.data_ptr() == out.data_ptr()
+    ref = np.concatenate([po.patchify(im, mean=mean, std=std, scale=scale)[0] for im in images])
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), ref.view(np.uint32))
+
+
+def test_patchify_full_benchmark_batch():
+    """The 8 ragged images of the benchmark workload (25,524 rows): bit-exact, and a still image fills both halves."""
+    _announce("patchify cfg2 batch")
+    grids = [[1, 76, 60], [1, 86, 54], [1, 82, 34], [1, 42, 78], [1, 54, 32], [1, 72, 56], [1, 40, 42], [1, 64, 44]]
+    images = _batch(4, [(1, 14 * h, 14 * w) for _, h, w in grids])
+    got, grid = _run(images)
+    assert grid.tolist() == grids and got.shape == (25524, 1176)
+    ref, _ = po.patchify_batch(images)
+    assert np.array_equal(got.numpy().view(np.uint32), ref.view(np.uint32))
+    halves = got.view(-1, 3, 2, 196)
+    assert torch.equal(halves[:, :, 0], halves[:, :, 1])
+
+
+def test_patchify_feeds_the_tower():
+    """pixel_values made on the GPU give the same tower output as the oracle's rows (same bits in, same bits out)."""
+    from mi355_vit.config import Qwen2_5_VLVisionConfig
+    from mi355_vit.modeling import Qwen2_5_VisionTransformerPretrainedModel
+    from mi355_vit.pixels import patchify
+
+    _announce("patchify -> tower")
+    images = _batch(5, [(1, 56, 84), (2, 56, 56)])
+    cfg = Qwen2_5_VLVisionConfig(depth=2, hidden_size=256, intermediate_size=300, num_heads=8, out_hidden_size=256,
+                                 window_size=56, fullatt_block_indexes=[1])
+    torch.manual_seed(0)
+    tower = Qwen2_5_VisionTransformerPretrainedModel(cfg).to(torch.bfloat16).to(DEV)
+    pv, grid = patchify([torch.from_numpy(im).to(DEV) for im in images], dtype=torch.bfloat16)
+    ref_pv = torch.from_numpy(po.patchify_batch(images)[0]).to(DEV)  # float32: the tower casts it as its first step
+    with torch.no_grad():
+        a = tower(pv, grid)
+        b = tower(ref_pv, grid)
+    assert torch.equal(a, b)
+
+
+def test_patchify_rejects_what_it_cannot_do():
+    from mi355_vit.pixels import patchify
+
+    ok = torch.zeros(1, 28, 28, 3, dtype=torch.uint8, device=DEV)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        patchify([ok.cpu()])
+    with pytest.raises(ValueError, match="multiples of 28"):
+        patchify([torch.zeros(1, 30, 28, 3, dtype=torch.uint8, device=DEV)])
+    with pytest.raises(ValueError, match="uint8"):
+        patchify([ok.float()])
+    with pytest.raises(TypeError):
+        patchify([ok], dtype=torch.float16)
+    with pytest.raises(ValueError, match="no images"):
+        patchify([])
+    with pytest.raises(RuntimeError, match="contiguous"):
+        patchify([torch.zeros(1, 28, 56, 3, dtype=torch.uint8, device=DEV)[:, :, ::2]])
