@@ -205,6 +205,54 @@ def handoff_leg(n_vision: int, hidden: int, dtype, iters: int = 20):
             "kernel_bytes_gbs": round(moved / (ours_ms * 1e-3) / 1e9, 1), "torch_masked_scatter_fwd_bwd_ms": round(ref_ms, 3)}
 
 
+def input_leg(grid, dtype, iters: int = 20):
+    """The step before the tower's input (not part of `value`): decoded uint8 frames of the workload's images ->
+    pixel_values rows in the tower's dtype, one launch for the batch, against the same steps written with torch
+    ops on the same GPU (rescale, normalise, reshape / permute per image, concatenate, cast)."""
+    from mi355_vit.pixels import OPENAI_CLIP_MEAN, OPENAI_CLIP_STD, patchify
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    frames = [torch.randint(0, 256, (int(t), 14 * int(h), 14 * int(w), 3), generator=g, dtype=torch.uint8).to(dev)
+              for t, h, w in grid.tolist()]
+    rows = int(grid.prod(dim=1).sum())
+    out = torch.empty((rows, 1176), dtype=dtype, device=dev)
+    mean = torch.tensor(OPENAI_CLIP_MEAN, dtype=torch.float32, device=dev)
+    std = torch.tensor(OPENAI_CLIP_STD, dtype=torch.float32, device=dev)
+
+    def ours():
+        return patchify(frames, dtype=dtype, out=out)[0]
+
+    def torch_ops():
+        parts = []
+        for f in frames:
+            n, h, w, _ = f.shape
+            x = ((f.double() * (1.0 / 255.0)).float() - mean) / std
+            x = x.permute(0, 3, 1, 2)
+            if n % 2:
+                x = torch.cat([x, x[-1:]], dim=0)
+            x = x.reshape(x.shape[0] // 2, 2, 3, h // 28, 2, 14, w // 28, 2, 14).permute(0, 3, 6, 4, 7, 2, 1, 5, 8)
+            parts.append(x.reshape(-1, 1176))
+        return torch.cat(parts, dim=0).to(dtype)
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            fn()
+        torch.cuda.synchronize()
+        return 1000.0 * (time.perf_counter() - t0) / iters
+
+    assert torch.equal(ours(), torch_ops())
+    ours_ms, ref_ms = timed(ours), timed(torch_ops)
+    frame_bytes = sum(f.numel() for f in frames)
+    moved = frame_bytes + rows * 1176 * out.element_size()  # every input byte once, every output value once
+    return {"images": len(frames), "rows": rows, "frame_bytes": frame_bytes, "out_dtype": str(dtype).replace("torch.", ""),
+            "patchify_ms": round(ours_ms, 3), "algorithmic_gbs": round(moved / (ours_ms * 1e-3) / 1e9, 1),
+            "torch_ops_ms": round(ref_ms, 3)}
+
+
 def cpu_baseline(cfg_kw, grid, seed, dtype, budget_s: float = 25.0):
     """Eager oracle (the reference's per-segment path, fp32) on the host cores, on a bounded sample: the two
     smallest images of the batch through patch embed, one windowed and one full-attention block and the
@@ -262,7 +310,7 @@ def main() -> None:
     ap.add_argument("--single-stream", action="store_true",
                     help="run weight / bias gradients in line on the main stream instead of on the second stream (for profiler "
                          "runs: kernels then never share the GPU, so their traced durations are their own)")
-    ap.add_argument("--no-optimizer", action="store_true", help="skip the optimizer-step measurement (reported beside the metric, never inside it)")
+    ap.add_argument("--no-optimizer", action="store_true", help="skip the optimizer-step, hand-off and input-side measurements (reported beside the metric, never inside it)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain device copy of 1 GiB (8 launches) so that profiler byte counters can be scaled to a known size")
     args = ap.parse_args()
@@ -354,6 +402,10 @@ def main() -> None:
     if not args.no_optimizer:
         handoff = handoff_leg(S // 4, cfg_kw["out_hidden_size"], dtype)
 
+    input_side = None
+    if not args.no_optimizer:
+        input_side = input_leg(grid, dtype)
+
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(cfg_kw, grid, seed, dtype)
@@ -379,6 +431,7 @@ def main() -> None:
         "cpu_baseline": cpu,
         "optimizer_step": optimizer,
         "vision_text_handoff": handoff,
+        "input_side": input_side,
         "kernel_breakdown": breakdown,
     }
     print(json.dumps(result))

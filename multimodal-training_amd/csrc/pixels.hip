@@ -1,9 +1,9 @@
 // Decoded RGB frames (uint8) -> rows of pixel_values for gfx950: rescale, normalise and cut into 14x14x2 patches in
 // the row order the vision tower expects, for a whole batch of images and videos in one launch.  HBM-bound: every
-// output row is 1176 values (4704 bytes in fp32) made from 2 x 588 input bytes; the input is read through the
-// caches byte by byte (a patch row is 42 contiguous bytes), the output leaves as 16-byte (fp32) or 8-byte (bf16)
-// stores, one wave per row and the four rows of a 2x2 merge block per work-group, so that a work-group reads one
-// 28x28 pixel square.
+// output row is 1176 values (4704 bytes in fp32) made from 2 x 588 input bytes (588 for a still image, whose one
+// frame fills both halves); the input is read through the caches byte by byte (a patch row is 42 contiguous
+// bytes), the output leaves as 16-byte (fp32) or 8-byte (bf16) stores, one wave per row and the four rows of a
+// 2x2 merge block per work-group, so that a work-group reads one 28x28 pixel square.
 //
 // The arithmetic is that of the image processor the reference calls (transformers 4.57.0,
 // Qwen2VLImageProcessor._preprocess: rescale in float64 rounded to float32, then (x - mean) / std in float32
@@ -15,7 +15,6 @@ namespace {
 constexpr int PATCH = 14, TPS = 2, ROW = MVIT_PIXEL_ROW;
 constexpr int PLANE = PATCH * PATCH;   // 196 values of one (channel, frame) plane of a row
 constexpr int QUADS = PLANE / 4;       // 49 groups of four consecutive values per plane
-constexpr int ROW_QUADS = ROW / 4;     // 294
 
 struct Norm {
   double rescale;
@@ -43,6 +42,15 @@ template <typename TO>
 __global__ __launch_bounds__(256) void patchify_kernel(const mvit_image* __restrict__ images, int n_images, TO* __restrict__ out,
                                                        int64_t total_rows, Norm nm) {
 #pragma clang fp contract(off)
+  // a byte has 256 values: the work-group computes the result for each of them and each channel once (exact
+  // arithmetic, three divisions per thread) and every element of its rows is then a byte load and a table lookup
+  __shared__ float lut[3][256];
+#pragma unroll
+  for (int c = 0; c < 3; ++c) {
+    const float x = (float)((double)(int)threadIdx.x * nm.rescale);
+    lut[c][threadIdx.x] = (x - nm.mean[c]) / nm.std[c];
+  }
+  __syncthreads();
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= total_rows) return;
   const int lane = threadIdx.x & 63;
@@ -57,20 +65,30 @@ __global__ __launch_bounds__(256) void patchify_kernel(const mvit_image* __restr
   const int y0 = (hb * 2 + ((rem >> 1) & 1)) * PATCH, x0 = (wb * 2 + (rem & 1)) * PATCH;
   if (t * TPS >= im.frames) return;  // first_row entries that promise more rows than the frames give
   const int64_t line = (int64_t)im.width * 3, frame_bytes = line * im.height;
+  const int f0 = t * TPS, f1 = f0 + 1 < im.frames ? f0 + 1 : im.frames - 1;  // the last frame fills an odd count up
+  const uint8_t* src0 = im.pixels + f0 * frame_bytes + y0 * line + x0 * 3;
+  const uint8_t* src1 = im.pixels + f1 * frame_bytes + y0 * line + x0 * 3;
   TO* dst = out + row * ROW;
-  for (int g = lane; g < ROW_QUADS; g += 64) {
-    const int c = g / (TPS * QUADS), tt = (g / QUADS) % TPS, q = g % QUADS;
-    int f = t * TPS + tt;
-    if (f >= im.frames) f = im.frames - 1;
-    const uint8_t* src = im.pixels + f * frame_bytes + y0 * line + x0 * 3 + c;
-    float v[4];
+  for (int g = lane; g < 3 * QUADS; g += 64) {
+    const int c = g / QUADS, q = g % QUADS;
+    int off[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const int p = 4 * q + e, py = p / PATCH, px = p % PATCH;
-      const float x = (float)((double)src[py * line + px * 3] * nm.rescale);
-      v[e] = (x - nm.mean[c]) / nm.std[c];
+      const int p = 4 * q + e;
+      off[e] = (p / PATCH) * (int)line + (p % PATCH) * 3 + c;
     }
-    store4(dst + 4 * g, v);
+    float v0[4], v1[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v0[e] = lut[c][src0[off[e]]];
+    if (f1 != f0) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v1[e] = lut[c][src1[off[e]]];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v1[e] = v0[e];
+    }
+    store4(dst + (c * TPS + 0) * PLANE + 4 * q, v0);
+    store4(dst + (c * TPS + 1) * PLANE + 4 * q, v1);
   }
 }
 
