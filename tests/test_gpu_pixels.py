@@ -66,6 +66,23 @@ def test_patchify_every_byte_value_other_constants_and_out_argument():
     assert np.array_equal(got.cpu().numpy().view(np.uint32), ref.view(np.uint32))
 
 
+def test_patchify_frames_at_an_odd_address():
+    """Frame buffers that are views one byte into an allocation: no dword alignment, byte path of the staging."""
+    from mi355_vit.pixels import patchify
+
+    _announce("patchify misaligned frames")
+    images = _batch(6, [(1, 56, 28), (3, 28, 84)])
+    views = []
+    for im in images:
+        buf = torch.zeros(im.size + 1, dtype=torch.uint8, device=DEV)
+        buf[1:].copy_(torch.from_numpy(im).reshape(-1))
+        views.append(buf[1:].view(im.shape))
+        assert views[-1].data_ptr() % 4 == 1
+    got, _ = patchify(views)
+    ref, _ = po.patchify_batch(images)
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), ref.view(np.uint32))
+
+
 def test_patchify_full_benchmark_batch():
     """The 8 ragged images of the benchmark workload (25,524 rows): bit-exact, and a still image fills both halves."""
     _announce("patchify cfg2 batch")
