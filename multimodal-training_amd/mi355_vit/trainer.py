@@ -341,6 +341,15 @@ class BaseVisionTrainer(Trainer):
             sample_index = sample_index.item() if sample_index.numel() == 1 else sample_index.tolist()
         device = torch.device("cuda:0")
         batch = dict(batch)
+        if batch.get("pixel_values") is None and batch.get("frames") is not None:
+            # resized uint8 frames ([frames, H, W, 3] per image or video) instead of the processor's float rows:
+            # a fifth of the upload, and rescale / normalise / patchify run on the GPU in the model's dtype
+            from .pixels import patchify
+
+            frames = [f.to(device, non_blocking=True).contiguous() for f in batch["frames"]]
+            param_dtype = next(self.model.parameters()).dtype
+            batch["pixel_values"], batch["image_grid_thw"] = patchify(
+                frames, dtype=param_dtype if param_dtype in (torch.float32, torch.bfloat16) else torch.float32)
         batch["pixel_values"] = batch["pixel_values"].to(device, non_blocking=True)
         batch["image_grid_thw"] = batch["image_grid_thw"].to(device, non_blocking=True)
         vision_outputs = self._model_forward(batch)

@@ -116,6 +116,29 @@ def test_patchify_feeds_the_tower():
     assert torch.equal(a, b)
 
 
+def test_trainer_takes_frames_batches():
+    """VisionTrainer.forward_step with a batch of uint8 frames equals the same step fed the oracle's pixel_values."""
+    from mi355_vit.trainer import VisionTrainer
+
+    _announce("trainer with frames batches")
+    cfg = dict(seed=0, parallelism="none", dtype="bfloat16", autocast=False, learning_rate=1e-3, weight_decay=0.0,
+               warmup_ratio=0.0, warmup_steps=0, lr_scheduler_type="constant", num_iterations=2, max_grad_norm=1.0,
+               activation_checkpointing=False, model_name=None,
+               vision_config=dict(depth=2, hidden_size=256, intermediate_size=300, num_heads=8, out_hidden_size=256,
+                                  window_size=56, fullatt_block_indexes=[1]))
+    images = _batch(7, [(1, 56, 84), (3, 28, 56)])
+    rows, grid = po.patchify_batch(images)
+    outs = []
+    for batch in ({"frames": [torch.from_numpy(im) for im in images], "sample_index": torch.tensor([0])},
+                  {"pixel_values": torch.from_numpy(rows), "image_grid_thw": torch.from_numpy(grid), "sample_index": torch.tensor([0])}):
+        tr = VisionTrainer(cfg, rank=0)
+        tr.build_model()
+        tr.set_data_iterator([batch])
+        tr.initialize_trainer()
+        outs.append(tr.forward_step(0)["vision_embeddings"].detach().clone())
+    assert torch.equal(outs[0], outs[1])
+
+
 def test_patchify_rejects_what_it_cannot_do():
     from mi355_vit.pixels import patchify
 
