@@ -48,7 +48,7 @@ CFG1 = dict(depth=4, hidden_size=1280, intermediate_size=3420, num_heads=16, out
 
 
 def test_config1_fp32_parity():
-    """BASELINE config 1: reduced tower, fp32, 2 images of 224x224; outputs and all gradients within 1e-4."""
+    """Benchmark configuration 1: reduced tower, fp32, 2 images of 224x224; outputs and all gradients within 1e-4."""
     print("[case] config-1 fp32 tower", flush=True)
     model = _build(CFG1, 0, torch.float32)
     g = torch.Generator().manual_seed(0)
