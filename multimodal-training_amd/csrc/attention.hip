@@ -35,13 +35,25 @@ struct AttnParams {
 
 // Which segment and head this work-group serves.  Work per work-group grows with its segment's length, so
 // callers list long segments first: the short ones then fill the tail of the launch.
+//
+// seg_major = 2 (short segments, grid (1, n_seg, heads) with n_seg * heads a multiple of 8): a head's slice of a
+// token row is 160 bytes at head_dim 80, so the heads of one segment share their 128-byte lines.  Work-group ids
+// are dealt round-robin to the 8 XCDs; id i therefore takes work item (i % 8) * (total / 8) + i / 8 of the
+// head-fastest list, which puts all heads of a segment on one XCD at about the same time and lets its L2 serve
+// the shared lines (the natural order reads them from memory once per head).
 __device__ __forceinline__ void seg_and_head(const AttnParams& p, int& seg, int& h) {
-  const int pos = p.seg_major ? blockIdx.z : blockIdx.y;
-  h = p.seg_major ? blockIdx.y : blockIdx.z;
+  int pos = p.seg_major == 1 ? blockIdx.z : blockIdx.y;
+  h = p.seg_major == 1 ? blockIdx.y : blockIdx.z;
+  const int n_seg = p.seg_major == 1 ? gridDim.z : gridDim.y;
+  if (p.seg_major == 2) {
+    const int nh = gridDim.z, lin = blockIdx.y + n_seg * blockIdx.z;
+    const int w = (lin & 7) * ((n_seg * nh) >> 3) + (lin >> 3);
+    pos = w / nh;
+    h = w % nh;
+  }
   seg = pos;
   if (p.order) {
     const int listed = p.order[pos];
-    const int n_seg = p.seg_major ? gridDim.z : gridDim.y;
     if ((unsigned)listed < (unsigned)n_seg) seg = listed;  // an entry outside the list never becomes an address
   }
 }
@@ -1248,7 +1260,9 @@ int launch_fwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
   dim3 grid((unsigned)((max_seqlen + 64 * nw - 1) / (64 * nw)), (unsigned)n_seg, (unsigned)p.nheads);
   if (nw == 1 && ND <= 5) {
     // windows: two waves x 32 queries share the staged K / V tiles (more waves per CU hide the load latency)
-    if constexpr (ND <= 5) hipLaunchKernelGGL((attn_fwd_mfma<ND, 2, 64, false, 2, 4>), grid, 128, 0, s, p);
+    AttnParams pw = p;
+    if (grid.x == 1 && ((int64_t)n_seg * p.nheads) % 8 == 0) pw.seg_major = 2;  // heads of a segment together on one XCD
+    if constexpr (ND <= 5) hipLaunchKernelGGL((attn_fwd_mfma<ND, 2, 64, false, 2, 4>), grid, 128, 0, s, pw);
   } else if (nw == 1) hipLaunchKernelGGL((attn_fwd_mfma<ND, 1, 64, false>), grid, 64, 0, s, p);
   else if (nw == 2) hipLaunchKernelGGL((attn_fwd_mfma<ND, 2, 64, false>), grid, 128, 0, s, p);
   else if constexpr (ND <= 5) {
@@ -1272,7 +1286,9 @@ int launch_bwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
     dim3 grid(1, (unsigned)n_seg, (unsigned)p.nheads);
     if constexpr (ND <= 5) {
       // four waves x 16 rows: ~160 registers, three work-groups (12 waves) per CU to cover the load -> MFMA -> store latency
-      hipLaunchKernelGGL((attn_bwd_window_mfma<ND, 4, 2>), grid, 256, 0, s, p);  // computes delta itself
+      AttnParams pw = p;
+      if (((int64_t)n_seg * p.nheads) % 8 == 0) pw.seg_major = 2;  // heads of a segment together on one XCD
+      hipLaunchKernelGGL((attn_bwd_window_mfma<ND, 4, 2>), grid, 256, 0, s, pw);  // computes delta itself
     } else {
       hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 1, 4>), grid, 64, 0, s, p);
       hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 1, 4>), grid, 64, 0, s, p);
