@@ -82,3 +82,18 @@ def test_batch_concatenates_like_the_collator_and_rejects_unresized_frames():
     assert np.array_equal(rows[:8], po.patchify(a)[0]) and np.array_equal(rows[8:], po.patchify(b)[0])
     with pytest.raises(AssertionError):
         po.patchify(_frames(7, 1, 30, 28))
+
+
+def test_host_mirror_grid_and_guards_without_a_gpu():
+    """mi355_vit.pixels: the grid it reports equals the oracle's, and what it cannot do is refused before any launch."""
+    from mi355_vit import pixels
+
+    frames = [torch.zeros(f, h, w, 3, dtype=torch.uint8) for f, h, w in [(1, 56, 84), (3, 28, 112), (4, 140, 28)]]
+    assert pixels.grid_thw_of(frames).tolist() == [list(po.grid_of(*f.shape[:3])) for f in frames]
+    assert pixels.OPENAI_CLIP_MEAN == po.OPENAI_CLIP_MEAN and pixels.OPENAI_CLIP_STD == po.OPENAI_CLIP_STD
+    for bad in (torch.zeros(1, 30, 28, 3, dtype=torch.uint8), torch.zeros(1, 28, 28, 4, dtype=torch.uint8),
+                torch.zeros(28, 28, 3, dtype=torch.uint8), torch.zeros(1, 28, 28, 3), torch.zeros(0, 28, 28, 3, dtype=torch.uint8)):
+        with pytest.raises(ValueError):
+            pixels.grid_thw_of([bad])
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        pixels.patchify(frames[:1])
