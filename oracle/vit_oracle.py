@@ -23,11 +23,18 @@ What pins each function (independently of this file's own formulae):
 ``attention``        ``F.scaled_dot_product_attention`` per segment
 ``mlp`` / ``merger`` ``F.silu`` / ``F.gelu`` / ``F.linear`` library routines
 ``patch_embed``      ``F.conv3d`` with kernel == stride vs. the GEMM form
-``tower_forward``    output shape [192, 256] of the reference's smoke test
-                     (tests/test_ragged_sp_smoke.py:27-98); numerics of the
-                     whole tower are **parity unpinned** by the reference (it
-                     holds no golden vectors for them) -- every arithmetic
-                     step is pinned piecewise as listed above.
+``attn_block``       vectors written by the reference's own module
+``block``            (tests/golden/reference_vectors.npz, made by
+``tower_forward``    tests/golden/make_reference_vectors.py from an import of
+                     modeling_qwen2_5_vl.py): output and every parameter
+                     gradient of a 3-layer tower on ragged / video grids,
+                     one attention module and one block alone, and the
+                     configuration-1 tower (default initialisation, seed 0);
+                     tests/test_oracle_golden.py also shows that the vectors
+                     reject rotary-on-V, a wrong segment list, an unpermuted
+                     rotary table and a missing reverse permutation, and
+                     checks the zero-angle / depth-0 special cases against
+                     ``F.multi_head_attention_forward`` and the bare merger.
 ===================  =========================================================
 """
 
@@ -279,3 +286,13 @@ def max_rel_err(a: torch.Tensor, b: torch.Tensor) -> float:
     if denom == 0.0:
         return (a - b).abs().max().item()
     return ((a - b).abs().max() / denom).item()
+
+
+def rel_frobenius_err(a: torch.Tensor, b: torch.Tensor) -> float:
+    """||a-b||_F / ||b||_F: a second metric beside max_rel_err, sensitive to errors spread over many small entries."""
+    a = a.detach().double().cpu()
+    b = b.detach().double().cpu()
+    denom = b.norm().item()
+    if denom == 0.0:
+        return (a - b).norm().item()
+    return ((a - b).norm() / denom).item()
