@@ -227,7 +227,15 @@ typedef struct {
   float step_size;
   float bias_correction2_sqrt;
   float weight_decay; /* L2 term: grad + weight_decay * param, as torch.optim.Adam (not decoupled) */
-  float reserved;
+  float unused;
+  /* Optional second destination of the updated parameter (NULL: none): the operand copy the GEMMs read (a fused
+   * q|k|v or gate|up weight, a weight with padded rows, a bf16 copy of an fp32 master weight).  The parameter is
+   * seen as rows of shadow_cols elements and element (row, col) is also stored at shadow[row * shadow_ld + col]
+   * (shadow_cols == 0: one row, i.e. a plain copy).  shadow_dtype is `dtype` or MVIT_BF16.  Only mvit_adam_step
+   * reads these fields. */
+  void* shadow;
+  int64_t shadow_cols, shadow_ld;
+  int32_t shadow_dtype, unused2;
 } mvit_adam_tensor;
 
 /* torch.optim.Adam(foreach=False, amsgrad=False, maximize=False) for every tensor of the table in one launch:

@@ -35,6 +35,49 @@ __device__ __forceinline__ int find_tensor(const mvit_adam_tensor* t, int n_tens
 template <typename T>
 __device__ __forceinline__ float rs(float x) { return to_f32(from_f32<T>(x)); }
 
+// Second copy of an updated parameter ("shadow"): the operand buffer the GEMMs read, in its own dtype and with its
+// own row pitch.  Element e of the parameter, seen as rows of `cols` elements, lands at shadow[row * ld + col].
+template <typename TS>
+__device__ __forceinline__ void shadow_store(void* shadow, int64_t e0, int n, int64_t cols, int64_t ld, const float* vals) {
+  TS* S = static_cast<TS*>(shadow);
+  int64_t idx = e0;
+  int64_t run = n;
+  if (cols != ld) {
+    const int64_t row = e0 / cols, col = e0 - row * cols;
+    idx = row * ld + col;
+    run = cols - col;
+  }
+  constexpr int V = mvit_elem<TS>::vec;
+  if (run >= n && n == V) {  // one contiguous piece: 16-byte store, or two 8-byte halves, by the address's alignment
+    typedef __attribute__((ext_vector_type(V))) TS vec_t;
+    typedef __attribute__((ext_vector_type(V / 2))) TS half_t;
+    vec_t out;
+#pragma unroll
+    for (int j = 0; j < V; ++j) out[j] = from_f32<TS>(vals[j]);
+    const uintptr_t a = reinterpret_cast<uintptr_t>(S + idx);
+    if ((a & 15u) == 0) {
+      *reinterpret_cast<vec_t*>(S + idx) = out;
+      return;
+    }
+    if ((a & 7u) == 0) {
+      half_t lo, hi;
+#pragma unroll
+      for (int j = 0; j < V / 2; ++j) {
+        lo[j] = out[j];
+        hi[j] = out[j + V / 2];
+      }
+      *reinterpret_cast<half_t*>(S + idx) = lo;
+      *reinterpret_cast<half_t*>(S + idx + V / 2) = hi;
+      return;
+    }
+  }
+  for (int j = 0; j < n; ++j) {  // pieces that wrap to the next row, odd tails, unaligned targets
+    const int64_t e = e0 + j;
+    const int64_t d = cols != ld ? (e / cols) * ld + (e % cols) : e;
+    S[d] = from_f32<TS>(vals[j]);
+  }
+}
+
 template <typename T>
 __device__ __forceinline__ void adam_elem(float& p, float& g, float& m, float& v, const AdamConsts& c, float wd,
                                           float neg_step_size, float bc2_sqrt) {
@@ -68,6 +111,8 @@ __global__ __launch_bounds__(NT) void adam_multi_kernel(const mvit_adam_tensor* 
   T* Vv = static_cast<T*>(t.exp_avg_sq) + base;
   const float wd = t.weight_decay, nss = -t.step_size, bc2 = t.bias_correction2_sqrt;
   const bool wg = c.write_grad && c.grad_scale != 1.0f;
+  const int64_t sh_cols = t.shadow_cols > 0 ? t.shadow_cols : t.numel, sh_ld = t.shadow_cols > 0 ? t.shadow_ld : t.numel;
+  const bool sh_bf16 = t.shadow_dtype == MVIT_BF16;
   const uintptr_t mis = (reinterpret_cast<uintptr_t>(P) | reinterpret_cast<uintptr_t>(G) | reinterpret_cast<uintptr_t>(M) |
                          reinterpret_cast<uintptr_t>(Vv)) & 15u;
   int done = 0;
@@ -76,10 +121,12 @@ __global__ __launch_bounds__(NT) void adam_multi_kernel(const mvit_adam_tensor* 
     for (int i = threadIdx.x; i < nvec; i += NT) {
       vec_t p = reinterpret_cast<vec_t*>(P)[i], g = reinterpret_cast<const vec_t*>(G)[i];
       vec_t m = reinterpret_cast<vec_t*>(M)[i], v = reinterpret_cast<vec_t*>(Vv)[i];
+      float pnew[V];
 #pragma unroll
       for (int j = 0; j < V; ++j) {
         float pf = to_f32(p[j]), gf = to_f32(g[j]), mf = to_f32(m[j]), vf = to_f32(v[j]);
         adam_elem<T>(pf, gf, mf, vf, c, wd, nss, bc2);
+        pnew[j] = pf;
         p[j] = from_f32<T>(pf);
         g[j] = from_f32<T>(gf);
         m[j] = from_f32<T>(mf);
@@ -89,6 +136,10 @@ __global__ __launch_bounds__(NT) void adam_multi_kernel(const mvit_adam_tensor* 
       reinterpret_cast<vec_t*>(M)[i] = m;
       reinterpret_cast<vec_t*>(Vv)[i] = v;
       if (wg) reinterpret_cast<vec_t*>(G)[i] = g;
+      if (t.shadow) {
+        if (sh_bf16) shadow_store<bf16_t>(t.shadow, base + (int64_t)i * V, V, sh_cols, sh_ld, pnew);  // fp32 parameters: element-wise
+        else shadow_store<float>(t.shadow, base + (int64_t)i * V, V, sh_cols, sh_ld, pnew);
+      }
     }
     done = nvec * V;
   }
@@ -99,6 +150,10 @@ __global__ __launch_bounds__(NT) void adam_multi_kernel(const mvit_adam_tensor* 
     M[i] = from_f32<T>(mf);
     Vv[i] = from_f32<T>(vf);
     if (wg) G[i] = from_f32<T>(gf);
+    if (t.shadow) {
+      if (sh_bf16) shadow_store<bf16_t>(t.shadow, base + i, 1, sh_cols, sh_ld, &pf);
+      else shadow_store<float>(t.shadow, base + i, 1, sh_cols, sh_ld, &pf);
+    }
   }
 }
 
@@ -163,6 +218,7 @@ int check_table(const char* what, const mvit_adam_tensor* tensors, int n_tensors
   MVIT_REQUIRE(tensors != nullptr && n_tensors > 0, "%s: empty tensor table", what);
   MVIT_REQUIRE(n_chunks > 0 && n_chunks <= 0x7fffffffLL, "%s: n_chunks %lld out of range", what, (long long)n_chunks);
   MVIT_REQUIRE(dtype == MVIT_BF16 || dtype == MVIT_F32, "%s: dtype %d", what, dtype);
+  static_assert(sizeof(mvit_adam_tensor) == 96, "table rows are 96 bytes");
   return MVIT_OK;
 }
 

@@ -37,7 +37,8 @@ class AdamTensor(C.Structure):
     _fields_ = [
         ("param", _vp), ("grad", _vp), ("exp_avg", _vp), ("exp_avg_sq", _vp),
         ("numel", _i64), ("first_chunk", _i64),
-        ("step_size", _f32), ("bias_correction2_sqrt", _f32), ("weight_decay", _f32), ("reserved", _f32),
+        ("step_size", _f32), ("bias_correction2_sqrt", _f32), ("weight_decay", _f32), ("unused", _f32),
+        ("shadow", _vp), ("shadow_cols", _i64), ("shadow_ld", _i64), ("shadow_dtype", _i32), ("unused2", _i32),
     ]
 
 

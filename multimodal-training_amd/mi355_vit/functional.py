@@ -46,6 +46,7 @@ class BlockWeights:
     C: int
     I: int
     Ipad: int
+    alias: bool = False  # norm1 / norm2 / wproj / bproj / bdown are the parameters themselves (same dtype), not copies
 
 
 # order of the parameter tensors handed to VisionBlockFn
@@ -59,30 +60,47 @@ BLOCK_PARAM_ORDER = (
 
 
 def pack_block_weights(params: List[torch.Tensor], dtype: torch.dtype, into: Optional[BlockWeights]) -> BlockWeights:
-    """(Re)fill the packed operands from the 16 parameters (cast to `dtype` on the way)."""
+    """(Re)fill the packed operands from the 16 parameters (cast to `dtype` on the way).
+
+    Operands that are a single parameter (norm weights, proj, the down bias) are the parameter itself when it
+    already has the compute dtype; the fused ones (q|k|v, gate|up, the padded down weight) are copies.  Every copy is
+    declared to the optimizer (``optim.attach_shadow``): ``FusedAdam.step`` writes updated values into it directly, so
+    an optimizer step never forces a re-pack; any other in-place change of a parameter bumps its version counter and
+    the owner of the pack calls this function again."""
+    from .optim import attach_shadow
+
     (n1, n2, wq, bq, wk, bk, wv, bv, wp, bp, wg, bg, wu, bu, wd, bd) = params
     C = wq.shape[1]
     I = wg.shape[0]
     Ipad = round_up(I, 8)
     dev = wq.device
-    if into is None or into.wqkv.dtype != dtype or into.wqkv.device != dev:
+    alias = all(p.dtype == dtype and p.is_contiguous() for p in (n1, n2, wp, bp, bd))
+    if into is None or into.wqkv.dtype != dtype or into.wqkv.device != dev or into.alias != alias:
         z = lambda *s: torch.zeros(*s, dtype=dtype, device=dev)  # noqa: E731
-        into = BlockWeights(z(1, C), z(1, C), z(3 * C, C), z(1, 3 * C), z(C, C), z(1, C), z(2 * Ipad, C), z(1, 2 * Ipad),
-                            z(C, Ipad), z(1, C), C, I, Ipad)
+        e = (lambda *s: None) if alias else z  # noqa: E731
+        into = BlockWeights(e(1, C), e(1, C), z(3 * C, C), z(1, 3 * C), e(C, C), e(1, C), z(2 * Ipad, C), z(1, 2 * Ipad),
+                            z(C, Ipad), e(1, C), C, I, Ipad, alias)
     cp = ops.cast2d
     v = lambda t: t.detach().view(1, -1)  # noqa: E731
-    cp(v(n1), into.norm1)
-    cp(v(n2), into.norm2)
+
+    def fill(param: torch.Tensor, dst: torch.Tensor) -> None:
+        cp(param.detach() if param.dim() == 2 else v(param), dst)
+        attach_shadow(param, dst if param.dim() == 2 else dst.view(-1))
+
+    if alias:
+        into.norm1, into.norm2, into.wproj, into.bproj, into.bdown = v(n1), v(n2), wp.detach(), v(bp), v(bd)
+        for param in (n1, n2, wp, bp, bd):
+            param._mvit_shadow = None  # read in place: nothing to keep in step
+    else:
+        for param, dst in ((n1, into.norm1), (n2, into.norm2), (wp, into.wproj), (bp, into.bproj), (bd, into.bdown)):
+            fill(param, dst)
     for j, (w, b) in enumerate(((wq, bq), (wk, bk), (wv, bv))):
-        cp(w.detach(), into.wqkv[j * C : (j + 1) * C])
-        cp(v(b), into.bqkv[:, j * C : (j + 1) * C])
-    cp(wp.detach(), into.wproj)
-    cp(v(bp), into.bproj)
+        fill(w, into.wqkv[j * C : (j + 1) * C])
+        fill(b, into.bqkv[:, j * C : (j + 1) * C])
     for j, (w, b) in enumerate(((wg, bg), (wu, bu))):
-        cp(w.detach(), into.wgu[j * Ipad : j * Ipad + I])
-        cp(v(b), into.bgu[:, j * Ipad : j * Ipad + I])
-    cp(wd.detach(), into.wdown[:, :I])
-    cp(v(bd), into.bdown)
+        fill(w, into.wgu[j * Ipad : j * Ipad + I])
+        fill(b, into.bgu[:, j * Ipad : j * Ipad + I])
+    fill(wd, into.wdown[:, :I])
     return into
 
 

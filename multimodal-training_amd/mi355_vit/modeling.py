@@ -127,7 +127,9 @@ class Qwen2_5_VLVisionBlock(nn.Module):
         return [self.get_parameter(n) for n in BLOCK_PARAM_ORDER]
 
     def packed(self, dtype: torch.dtype):
-        """Packed compute-dtype operands, refreshed when a parameter was modified (optimizer step, load)."""
+        """Packed compute-dtype operands.  They are rebuilt when a parameter was replaced or modified in place
+        through torch (load_state_dict, a torch optimizer: the version counter moves); FusedAdam updates parameters
+        through raw pointers and writes the packed copies itself in the same pass, so its steps need no rebuild."""
         params = self._block_params()
         key = (dtype,) + tuple((p.data_ptr(), p._version) for p in params)
         if key != self._packed_key:

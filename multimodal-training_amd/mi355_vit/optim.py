@@ -24,9 +24,31 @@ from . import _lib
 
 _TABLE_DTYPE = np.dtype(
     [("param", "<u8"), ("grad", "<u8"), ("exp_avg", "<u8"), ("exp_avg_sq", "<u8"), ("numel", "<i8"), ("first_chunk", "<i8"),
-     ("step_size", "<f4"), ("bias_correction2_sqrt", "<f4"), ("weight_decay", "<f4"), ("reserved", "<f4")]
+     ("step_size", "<f4"), ("bias_correction2_sqrt", "<f4"), ("weight_decay", "<f4"), ("unused", "<f4"),
+     ("shadow", "<u8"), ("shadow_cols", "<i8"), ("shadow_ld", "<i8"), ("shadow_dtype", "<i4"), ("unused2", "<i4")]
 )
-assert _TABLE_DTYPE.itemsize == C.sizeof(_lib.AdamTensor) == 64
+assert _TABLE_DTYPE.itemsize == C.sizeof(_lib.AdamTensor) == 96
+_NO_SHADOW = (0, 0, 0, 0, 0)
+
+
+def attach_shadow(param: torch.Tensor, copy: torch.Tensor) -> None:
+    """Declare ``copy`` (a 1-D or 2-D view with unit column stride, of the parameter's dtype or bfloat16) the operand
+    copy of ``param`` that the kernels read: ``FusedAdam.step`` then stores every updated element there as well, so
+    the copy never has to be rebuilt after a step.  ``copy`` must have the parameter's shape."""
+    if copy.shape != param.shape or copy.dim() not in (1, 2) or copy.stride(-1) != 1 or copy.device != param.device:
+        raise ValueError("attach_shadow: the copy must be a 1-D / 2-D unit-stride view of the parameter's shape on its device")
+    if copy.dtype not in (param.dtype, torch.bfloat16):
+        raise ValueError("attach_shadow: the copy's dtype must be the parameter's or bfloat16")
+    param._mvit_shadow = copy
+
+
+def _shadow_fields(p: torch.Tensor) -> tuple:
+    sh = getattr(p, "_mvit_shadow", None)
+    if sh is None:
+        return _NO_SHADOW
+    cols = sh.shape[-1]
+    ld = sh.stride(0) if sh.dim() == 2 else cols
+    return (sh.data_ptr(), cols, ld, _dtype_code(sh.dtype), 0)
 
 
 def _check_tensor(t: torch.Tensor, what: str) -> None:
@@ -118,7 +140,7 @@ class FusedAdam(torch.optim.Adam):
                     bk.group_slices.append([gi, len(bk.rows), len(bk.rows)])
                 bk.params.append(p)
                 bk.step_tensors.append(st["step"])
-                bk.rows.append((p.data_ptr(), 0, m.data_ptr(), v.data_ptr(), p.numel(), 0, 0.0, 0.0, 0.0, 0.0))
+                bk.rows.append((p.data_ptr(), 0, m.data_ptr(), v.data_ptr(), p.numel(), 0, 0.0, 0.0, 0.0, 0.0) + _shadow_fields(p))
                 bk.group_slices[-1][2] = len(bk.rows)
         for bk in buckets.values():
             bk.finish()
@@ -134,7 +156,7 @@ class FusedAdam(torch.optim.Adam):
                 loss = closure()
         # which parameters take part (those with a gradient) and where they and their moments live rarely changes:
         # the table is rebuilt only when it does; per step only gradient addresses and scalars are refreshed
-        key = tuple((id(p), p.data_ptr()) for group in self.param_groups for p in group["params"] if p.grad is not None)
+        key = tuple((id(p), p.data_ptr(), _shadow_fields(p)) for group in self.param_groups for p in group["params"] if p.grad is not None)
         stale = key != self._plan_key or any(
             int(bk.step_tensors[0].item()) != int(bk.steps[0]) or int(bk.step_tensors[-1].item()) != int(bk.steps[-1])
             for bk in self._plan)  # step counters edited from outside (cheap spot check of the host mirror)
@@ -193,7 +215,7 @@ def grad_norm_squared(params: Iterable[torch.Tensor]) -> float:
         if g is None or g.numel() == 0:
             continue
         _check_tensor(g, "grad_norm_squared gradient")
-        buckets.setdefault((g.device, g.dtype), []).append((0, g.data_ptr(), 0, 0, g.numel(), 0, 0.0, 0.0, 0.0, 0.0))
+        buckets.setdefault((g.device, g.dtype), []).append((0, g.data_ptr(), 0, 0, g.numel(), 0, 0.0, 0.0, 0.0, 0.0) + _NO_SHADOW)
     lib = _lib.load()
     outs = []
     for (device, dtype), rows in buckets.items():

@@ -178,3 +178,51 @@ def test_trainer_uses_the_multi_tensor_step():
                                     weight_decay=wd, grad_scale=coeff)
         assert torch.equal(p.detach().cpu(), ref["param"]), n
         assert torch.equal(p.grad.cpu(), ref["grad"]), n
+
+
+@pytest.mark.parametrize("dtype,copy_dtype", [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32), (torch.float32, torch.bfloat16)])
+def test_fused_adam_keeps_operand_copies_in_step(dtype, copy_dtype):
+    """Parameters with a declared operand copy (plain, row-padded, at an offset inside a fused buffer, odd sizes):
+    after every step the copy holds exactly the updated parameter (rounded once when the copy is bf16), the
+    padding columns stay untouched, and the parameters equal those of a run without copies bit for bit."""
+    from mi355_vit.optim import FusedAdam, attach_shadow
+
+    _announce(f"operand copies {dtype} -> {copy_dtype}")
+    g = torch.Generator().manual_seed(11)
+    shapes = [(64, 3420), (300, 257), (1280,), (5, 7), (8192 * 2 + 3,), (96, 40)]
+    params = [(torch.randn(s, generator=g) * 0.05).to(dtype) for s in shapes]
+    plain = [torch.nn.Parameter(p.to(DEV)) for p in params]
+    shadowed = [torch.nn.Parameter(p.to(DEV)) for p in params]
+    bufs, views = [], []
+    for i, p in enumerate(shadowed):
+        if p.dim() == 2:
+            pad = (0, 4, 7, 0, 0, 8)[i]
+            buf = torch.full((p.shape[0] + 3, p.shape[1] + pad), 77.0, dtype=copy_dtype, device=DEV)
+            view = buf[2 : 2 + p.shape[0], : p.shape[1]]
+        else:
+            buf = torch.full((p.numel() + 5,), 77.0, dtype=copy_dtype, device=DEV)
+            view = buf[(0, 0, 4, 0, 1, 0)[i] :][: p.numel()]
+        view.copy_(p.detach())
+        attach_shadow(p, view)
+        bufs.append(buf)
+        views.append(view)
+    o1, o2 = FusedAdam(plain, lr=1e-2, weight_decay=0.01), FusedAdam(shadowed, lr=1e-2, weight_decay=0.01)
+    for step in range(3):
+        for a, b in zip(plain, shadowed):
+            gr = (torch.randn(a.shape, generator=g) * 0.1).to(dtype).to(DEV)
+            a.grad, b.grad = gr, gr.clone()
+        o1.step(grad_scale=0.5)
+        o2.step(grad_scale=0.5)
+        torch.cuda.synchronize()
+        for a, b, view, buf in zip(plain, shadowed, views, bufs):
+            assert torch.equal(a.detach(), b.detach())
+            assert torch.equal(view, b.detach().to(copy_dtype))
+            mask = torch.ones_like(buf, dtype=torch.bool)
+            if buf.dim() == 2:
+                mask[2 : 2 + b.shape[0], : b.shape[1]] = False
+            else:
+                off = view.data_ptr() - buf.data_ptr()
+                mask[off // buf.element_size() :][: b.numel()] = False
+            assert bool((buf[mask] == 77.0).all()), "the step wrote outside the copy"
+    with pytest.raises(ValueError):
+        attach_shadow(shadowed[0], torch.zeros(3, 3, device=DEV, dtype=copy_dtype))

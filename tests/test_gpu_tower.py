@@ -215,3 +215,57 @@ def test_trainer_fifo_and_checkpoint_roundtrip(tmp_path):
     for k, v in tr.model.state_dict().items():
         assert torch.equal(v.cpu(), sd[k]), k
     assert not tr.load_checkpoint(str(tmp_path), epoch=9)
+
+
+@pytest.mark.parametrize("dtype,autocast", [(torch.bfloat16, False), (torch.float32, False), (torch.float32, True)])
+def test_forward_after_a_fused_adam_step_uses_the_updated_weights(dtype, autocast):
+    """The step writes parameters through raw pointers (no version counter moves): the packed operands the blocks
+    read must follow anyway.  Same input before and after one step; the second output must match the oracle run on
+    the updated parameters and differ from the first output."""
+    from mi355_vit.optim import FusedAdam
+
+    print(f"[case] forward after FusedAdam step {dtype} autocast={autocast}", flush=True)
+    kw = dict(depth=2, hidden_size=256, intermediate_size=300, num_heads=8, out_hidden_size=128, fullatt_block_indexes=[1])
+    model = _build(kw, 5, dtype).to(DEV).train()
+    g = torch.Generator().manual_seed(5)
+    grid = torch.tensor([[1, 16, 16], [1, 8, 24]])
+    S = 16 * 16 + 8 * 24
+    pixels = torch.randn(S, 1176, generator=g).to(DEV)
+    gout = torch.randn(S // 4, 128, generator=g).to(DEV)
+    # gradients for the block parameters only: a change of the output can then only come from the blocks
+    block_params = [p for n, p in model.named_parameters() if n.startswith("blocks.")]
+    opt = FusedAdam(block_params, lr=5e-3, weight_decay=0.01)
+
+    def forward():
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+            return model(hidden_states=pixels, grid_thw=grid.to(DEV))
+
+    outs = []
+    for step in range(3):
+        out = forward()
+        outs.append(out.detach().float().cpu())
+        model.zero_grad(set_to_none=True)
+        out.backward(gout.to(out.dtype))
+        for n, p in model.named_parameters():
+            if not n.startswith("blocks."):
+                p.grad = None
+        opt.step()
+    final = forward().detach().float().cpu()
+    torch.cuda.synchronize()
+    assert max_rel_err(final, outs[0]) > 5e-2, "three optimizer steps left the output unchanged: stale operands"
+    assert max_rel_err(outs[1], outs[0]) > 1e-2
+    low = dtype == torch.bfloat16 or autocast
+    cpu = copy.deepcopy(model).cpu()
+    params = {k: (v.detach().to(torch.bfloat16).float() if low else v.detach().float()).clone() for k, v in cpu.state_dict().items()}
+    inv_freq = cpu.rotary_pos_emb.inv_freq.detach().clone()
+    with torch.no_grad():
+        ref = vit_oracle.tower_forward(pixels.cpu().float(), grid, params, _oracle_cfg(kw), inv_freq=inv_freq)
+    assert max_rel_err(final, ref) < (2e-2 if low else 1e-4)
+    # a torch optimizer (in-place torch ops) on the same parameters is followed as well
+    sgd = torch.optim.SGD(block_params, lr=0.5)
+    out = forward()
+    model.zero_grad(set_to_none=True)
+    out.backward(gout.to(out.dtype))
+    sgd.step()
+    after_sgd = forward().detach().float().cpu()
+    assert max_rel_err(after_sgd, final) > 1e-2
