@@ -258,6 +258,17 @@ int mvit_adam_step(const mvit_adam_tensor* tensors, int n_tensors, int64_t n_chu
 int mvit_grad_sumsq(const mvit_adam_tensor* tensors, int n_tensors, int64_t n_chunks, float* partial, double* out,
                     int dtype, mvit_stream_t stream);
 
+/* mvit_grad_sumsq without the workspace argument, for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight loops, harnesses that forbid hipMalloc): the per-chunk partial sums live in an array
+ * built into the library (MVIT_SUMSQ_STATIC_MAX_CHUNKS floats = 1 MiB per GPU, held until the process ends).  It
+ * has no counterpart in the reference.  Same results as mvit_grad_sumsq, bit for bit.  n_chunks above the maximum
+ * is rejected with MVIT_ERR_ARG.  The first call on a device looks up the array's address (no allocation); no call
+ * allocates or frees memory.  All calls on one GPU share the array: calls that overlap in time on one GPU (two
+ * streams, two threads) race and must be serialised by the caller. */
+#define MVIT_SUMSQ_STATIC_MAX_CHUNKS 262144 /* x MVIT_ADAM_CHUNK = 2^31 elements */
+int mvit_grad_sumsq_static(const mvit_adam_tensor* tensors, int n_tensors, int64_t n_chunks, double* out, int dtype,
+                           mvit_stream_t stream);
+
 /* ---------------------------------------------------------------- input side: decoded frames -> pixel_values */
 
 #define MVIT_PIXEL_ROW 1176 /* 3 channels x 2 frames x 14 x 14: one row of pixel_values */

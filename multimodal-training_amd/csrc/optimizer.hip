@@ -11,6 +11,13 @@
 // addcdiv as a + (value * b) / c), with no other contraction, so fp32 results can be compared bit for bit.
 #include "mvit_common.h"
 
+#include <mutex>
+
+// Scratch of the entry point that allocates nothing (mvit_grad_sumsq_static): per-chunk partial sums.  Every GPU the
+// library runs on holds its own copy of this array until the process ends.  In host code the name is only a handle
+// for hipGetSymbolAddress; kernels and every other use take the device address looked up once per device.
+static __device__ __align__(256) float scratch[MVIT_SUMSQ_STATIC_MAX_CHUNKS];
+
 namespace {
 
 constexpr int CHUNK = MVIT_ADAM_CHUNK;
@@ -222,6 +229,28 @@ int check_table(const char* what, const mvit_adam_tensor* tensors, int n_tensors
   return MVIT_OK;
 }
 
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[MAX_DEVICES] = {};  // device address of `scratch` on each device, looked up on first use
+
+// Address of the current device's copy of `scratch` (set-up on the first call per device; no allocation).
+int static_scratch(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES)
+    return mvit_set_error(MVIT_ERR_LAUNCH, "grad_sumsq_static: hipGetDevice: %s (device %d)", hipGetErrorString(e), dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      return mvit_set_error(MVIT_ERR_LAUNCH, "grad_sumsq_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = static_cast<float*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return MVIT_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -261,6 +290,19 @@ int mvit_grad_sumsq(const mvit_adam_tensor* tensors, int n_tensors, int64_t n_ch
   hipLaunchKernelGGL(sumsq_final_kernel, dim3(1), 1024, 0, s, (const float*)partial, n_chunks, out);
   MVIT_CHECK_LAUNCH("grad_sumsq (final)");
   return MVIT_OK;
+}
+
+int mvit_grad_sumsq_static(const mvit_adam_tensor* tensors, int n_tensors, int64_t n_chunks, double* out, int dtype,
+                           mvit_stream_t stream) {
+  if (int rc = check_table("grad_sumsq_static", tensors, n_tensors, n_chunks, dtype)) return rc;
+  MVIT_REQUIRE(out != nullptr, "grad_sumsq_static: null output");
+  MVIT_REQUIRE(n_chunks <= (int64_t)MVIT_SUMSQ_STATIC_MAX_CHUNKS,
+               "grad_sumsq_static: %lld chunks exceed the built-in scratch of %d chunks (%lld elements); use mvit_grad_sumsq with a workspace",
+               (long long)n_chunks, MVIT_SUMSQ_STATIC_MAX_CHUNKS, (long long)MVIT_SUMSQ_STATIC_MAX_CHUNKS * MVIT_ADAM_CHUNK);
+  float* partial = nullptr;
+  if (int rc = static_scratch(&partial)) return rc;
+  // every partial in [0, n_chunks) is overwritten by the first kernel, so nothing has to be cleared between calls
+  return mvit_grad_sumsq(tensors, n_tensors, n_chunks, partial, out, dtype, stream);
 }
 
 }  // extern "C"

@@ -43,6 +43,7 @@ class AdamTensor(C.Structure):
 
 
 ADAM_CHUNK = 8192
+SUMSQ_STATIC_MAX_CHUNKS = 262144
 
 
 class Image(C.Structure):
@@ -75,6 +76,7 @@ PROTOTYPES = {
     "mvit_merge_rows": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "mvit_adam_step": [_vp, _i32, _i64, C.c_double, C.c_double, C.c_double, C.c_double, _i32, _i32, _vp],
     "mvit_grad_sumsq": [_vp, _i32, _i64, _vp, _vp, _i32, _vp],
+    "mvit_grad_sumsq_static": [_vp, _i32, _i64, _vp, _i32, _vp],
     "mvit_patchify": [_vp, _i32, _i64, _vp, C.c_double] + [_f32] * 6 + [_i32, _vp],
     "mvit_attn_bwd": [_vp] * 12 + [_i32, _i32, _i64, _i32, _i32] + [_i64] * 8 + [_f32, _i32, _vp],
 }

@@ -206,9 +206,10 @@ def _build_table(rows: List[tuple]) -> Tuple[np.ndarray, int]:
     return table, int(table["first_chunk"][n])
 
 
-def grad_norm_squared(params: Iterable[torch.Tensor]) -> float:
+def grad_norm_squared(params: Iterable[torch.Tensor], static_scratch: bool = False) -> float:
     """sum over parameters of ||grad||_2^2 (fp32 within a chunk of 8192 elements, fp64 across chunks): the quantity
-    Trainer._compute_grad_norm_squared returns, with one host read-back in total."""
+    Trainer._compute_grad_norm_squared returns, with one host read-back in total.  ``static_scratch`` keeps the
+    per-chunk partial sums in the array built into the library (mvit_grad_sumsq_static) instead of a fresh tensor."""
     buckets: Dict[tuple, List[tuple]] = {}
     for p in params:
         g = p.grad
@@ -221,12 +222,15 @@ def grad_norm_squared(params: Iterable[torch.Tensor]) -> float:
     for (device, dtype), rows in buckets.items():
         table, n_chunks = _build_table(rows)
         dev_table = _upload(table, device)
-        partial = torch.empty(n_chunks, dtype=torch.float32, device=device)
         out = torch.empty(1, dtype=torch.float64, device=device)
         with torch.cuda.device(device):
             stream = torch.cuda.current_stream(device).cuda_stream
-            rc = lib.mvit_grad_sumsq(dev_table.data_ptr(), len(rows), n_chunks, partial.data_ptr(), out.data_ptr(),
-                                     _dtype_code(dtype), stream)
+            if static_scratch:
+                rc = lib.mvit_grad_sumsq_static(dev_table.data_ptr(), len(rows), n_chunks, out.data_ptr(), _dtype_code(dtype), stream)
+            else:
+                partial = torch.empty(n_chunks, dtype=torch.float32, device=device)
+                rc = lib.mvit_grad_sumsq(dev_table.data_ptr(), len(rows), n_chunks, partial.data_ptr(), out.data_ptr(),
+                                         _dtype_code(dtype), stream)
         _lib.check(rc, "mvit_grad_sumsq")
         outs.append(out)
     if not outs:
