@@ -230,7 +230,11 @@ class VisionBlockFn(torch.autograd.Function):
         W = ctx.holder.packed(x.dtype)
         saved = ctx.saved
         if saved is None:
-            _, saved = _block_forward(x, W, geo, ctx.eps)
+            ops.recomputing = True
+            try:
+                _, saved = _block_forward(x, W, geo, ctx.eps)
+            finally:
+                ops.recomputing = False
         dx, grads = _block_backward(dx2, x, saved, W, geo, ctx.gdt)
         ctx.saved = None
         ctx.x = None

@@ -20,6 +20,7 @@ GEMM_PANEL = int(_os.environ.get("MI355_VIT_GEMM_PANEL", "0"))  # bits 0-7: tile
 GEMM_VARIANT = int(_os.environ.get("MI355_VIT_GEMM_VARIANT", "0"))  # GEMM main loop: 0 default, 1 register-staged, 3 direct-to-LDS, 5 / 7 one MFMA shape only
 
 _trace = None  # optional list collecting (tag, info, start_event, end_event) per tagged launch
+recomputing = False  # True while a checkpointed block re-runs its forward inside the backward (marks traced launches)
 
 
 def set_trace(records: Optional[list]) -> None:
@@ -51,7 +52,7 @@ def _launch(tag: str, info: dict, call):
     e0.record()
     rc = call()
     e1.record()
-    _trace.append((tag, info, e0, e1))
+    _trace.append((tag, dict(info, recompute=recomputing), e0, e1))
     return rc
 
 
