@@ -181,7 +181,9 @@ int mvit_attn_fwd(const void* q, const void* k, const void* v, void* o, float* l
                   int64_t k_stride, int64_t v_stride, int64_t o_stride, float scale, int dtype,
                   mvit_stream_t stream);
 
-/* Gradients of the above.  delta: fp32 workspace [nheads, total].  dq/dk/dv use the q/k/v strides given. */
+/* Gradients of the above.  delta: fp32 workspace [3, nheads, total] (row sums of o * d_o and two rescaled copies
+ * of the row statistics).  dq/dk/dv use the strides given and must not overlap any input: the dq buffer is also
+ * used as scratch (pre-scaled queries) before the result is written to it. */
 int mvit_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
                   void* dq, void* dk, void* dv, float* delta, const int32_t* cu_seqlens,
                   const int32_t* seg_order, int n_seg, int max_seqlen, int64_t total, int nheads, int head_dim, int64_t q_stride, int64_t k_stride,

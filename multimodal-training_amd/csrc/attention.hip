@@ -14,6 +14,8 @@
 // fp32 path (parity mode): one lane per query (or key) row, K/V (or Q/dO) tiles broadcast from LDS.
 #include "mvit_common.h"
 
+#include <algorithm>
+
 namespace {
 
 constexpr float LOG2E = 1.4426950408889634f;
@@ -29,6 +31,9 @@ struct AttnParams {
   int nheads;
   int64_t q_stride, k_stride, v_stride, o_stride, do_stride, dq_stride, dk_stride, dv_stride;
   float scale;
+  const void* q_scaled;  // wide backward: bf16(Q * scale * log2(e)), row stride qs_stride
+  int64_t qs_stride;
+  const float *nlse2, *ndelta;  // wide backward: - lse * log2(e) and - delta, [nheads, total]
   const int32_t* order;  // optional: the segment scheduled at grid position i is order[i] (null: i)
   int seg_major;         // 0: grid (x, segment, head); 1: grid (x, head, segment), all heads of a segment together
 };
@@ -495,6 +500,380 @@ __global__ __launch_bounds__(64 * NWAVES, MINW) void attn_fwd_mfma(const AttnPar
   }
 }
 
+// ================================================================================================
+// Long segments, "wide" kernels: a wave owns 64 rows (two 32-row blocks), four waves per work-group, one
+// work-group per CU (up to 512 registers per lane).  Products whose contraction runs over head_dim use
+// v_mfma_f32_32x32x16_bf16, so head_dim = 16 * ND is contracted exactly (80 = 5 x 16, no padding); products whose
+// contraction runs over rows (keys or queries) use v_mfma_f32_16x16x32_bf16 with head_dim as the 16-wide M dimension.
+// A 32x32 accumulator tile (lane: column l%32; register i: row 8*(i/4) + 4*(l/32) + i%4) becomes the B operand of the
+// 16x16x32 product after packing to bf16 pairs and four v_permlane16_swap: lanes l and l^16 exchange halves, after
+// which lane l holds, for columns l%16 (words 0-3) and 16 + l%16 (words 4-7), the rows
+//     base(G) + {0..3}  and  base(G) + 8 + {0..3},   G = l / 16,  base = {0, 16, 4, 20}[G]
+// in its eight contraction slots; the transposed left factor is read from LDS with the same row mapping.
+// Row statistics ride in the accumulator input of the first MFMA of a chain (a tile of "- stabiliser" values), so
+// exp2 is applied to the MFMA result directly.
+typedef unsigned int u32x8_t __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ f32x16 mfma32x32(const bf16x8& a, const bf16x8& b, const f32x16& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+// acc += a . b on v_mfma_f32_16x16x32_bf16 with the accumulator pinned to the accumulation registers (the compiler
+// otherwise moves accumulators between the two register files).  It does not see an MFMA here: before ordinary
+// instructions touch such an accumulator again, mfma_drain() must have run.
+__device__ __forceinline__ void mfma16_acc(f32x4& acc, const bf16x8& a, const bf16x8& b) {
+  acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+}
+// d = a . b + c and d += a . b on v_mfma_f32_32x32x16_bf16, all operands in ordinary vector registers (the compiler's own
+// MFMA selection would place results in accumulation registers and copy them back for the vector ALU).  The same rule
+// applies: ordinary instructions may read d only after mfma_drain() or after eleven or more other issue slots.
+// The B operand `b` sits in accumulation registers (see to_acc_regs): an operand that never changes costs no
+// ordinary register that way.
+__device__ __forceinline__ void mfma32x32_init(f32x16& d, const bf16x8& a, const u32x4& b, const f32x16& c) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(__builtin_bit_cast(u32x4, a)), "a"(b), "v"(c));
+}
+__device__ __forceinline__ void mfma32x32_acc(f32x16& d, const bf16x8& a, const u32x4& b) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(__builtin_bit_cast(u32x4, a)), "a"(b));
+}
+// Moves a fragment into accumulation registers through the lane's own 16-byte LDS slot (a DS load can target them).
+__device__ __forceinline__ u32x4 to_acc_regs(const bf16x8& v, float* slot) {
+  const unsigned addr = (unsigned)(uintptr_t)slot;
+  *reinterpret_cast<volatile bf16x8*>(slot) = v;
+  u32x4 r;
+  asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=a"(r) : "v"(addr) : "memory");
+  return r;
+}
+// acc *= factor for an accumulator that lives in the accumulation registers, without the compiler ever seeing it
+// in an ordinary register (it would then keep a second copy of every accumulator across the whole loop): the four
+// values travel through the lane's own 16-byte LDS slot.  Rare path only; call mfma_drain() first.
+__device__ __forceinline__ void scale_acc(f32x4& acc, float factor, float* slot) {
+  const unsigned addr = (unsigned)(uintptr_t)slot;  // LDS byte address
+  asm volatile("ds_write_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(addr), "a"(acc) : "memory");
+  f32x4 t = *reinterpret_cast<volatile f32x4*>(slot);
+  t *= factor;
+  *reinterpret_cast<volatile f32x4*>(slot) = t;
+  asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=a"(acc) : "v"(addr) : "memory");
+}
+__device__ __forceinline__ void mfma_drain() {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+__device__ __forceinline__ f32x16 splat16(float x) {
+  f32x16 r;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) r[i] = x;
+  return r;
+}
+__device__ __forceinline__ unsigned pack2(float a, float b) {
+  bf16x2 v = {(bf16_t)a, (bf16_t)b};
+  return __builtin_bit_cast(unsigned, v);
+}
+// lanes l and l^16 trade: afterwards a = the pair's value for the lower lane's column, b = for the upper lane's
+__device__ __forceinline__ void swap16(unsigned& a, unsigned& b) {
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap16f(float& a, float& b) {
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+// value held by lane l^32
+__device__ __forceinline__ float other_half(float x) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  return (threadIdx.x & 32) ? a : b;  // the swap put the partner's value into b of the lower half and a of the upper half
+}
+struct BOps {
+  bf16x8 lo, hi;  // B operands of the 16x16x32 product for columns l%16 and 16 + l%16 of the 32-column tile
+};
+__device__ __forceinline__ BOps to_b_operands(unsigned (&w)[8]) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) swap16(w[j], w[j + 4]);
+  const u32x4 a = {w[0], w[1], w[2], w[3]}, b = {w[4], w[5], w[6], w[7]};
+  BOps r;
+  r.lo = __builtin_bit_cast(bf16x8, a);
+  r.hi = __builtin_bit_cast(bf16x8, b);
+  return r;
+}
+// A operand (16 x 32, transposed read) of the 16x16x32 product matching to_b_operands: rows base(G)+.. of the
+// 32-row group starting at `row0` of a [row][PITCH] tile, columns 16*d .. 16*d+15.
+template <int PITCH>
+__device__ __forceinline__ bf16x8 tr_block_wide(const bf16_t* tile, int row0, int d, int G, int r) {
+  const int row = row0 + 16 * (G & 1) + 4 * (G >> 1) + (r >> 2);
+  if (PITCH == SWZ) {
+    const int chunk = 2 * d + ((r & 3) >> 1), sub = 4 * (r & 1);
+    return tr_pair(tile + swz_off(row, chunk) + sub, tile + swz_off(row + 8, chunk) + sub);
+  }
+  const bf16_t* a = tile + row * PITCH + 16 * d + 4 * (r & 3);
+  return tr_pair(a, a + 8 * PITCH);
+}
+// Row fragment (A or B operand of the 32x32x16 product) of row `row` of a [row][PITCH] tile: 8 elements at 16*s + 8*h.
+template <int PITCH>
+__device__ __forceinline__ bf16x8 row_frag32(const bf16_t* tile, int row, int s, int h) {
+  if (PITCH == SWZ) return *reinterpret_cast<const bf16x8*>(tile + swz_off(row, 2 * s + h));
+  return *reinterpret_cast<const bf16x8*>(tile + row * PITCH + 16 * s + 8 * h);
+}
+__device__ __forceinline__ bf16x8 scale_frag(bf16x8 v, float c) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = (bf16_t)((float)v[j] * c);
+  return v;
+}
+__device__ __forceinline__ bf16x8 load_frag_global(const bf16_t* p, bool valid) {
+  bf16x8 v;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = (bf16_t)0.f;
+  if (valid) v = *reinterpret_cast<const bf16x8*>(p);
+  return v;
+}
+__device__ __forceinline__ float max16(const f32x16& s) {
+  float m = max3(s[0], s[1], s[2]);
+  m = max3(m, s[3], s[4]);
+  m = max3(m, s[5], s[6]);
+  m = max3(m, s[7], s[8]);
+  m = max3(m, s[9], s[10]);
+  m = max3(m, s[11], s[12]);
+  m = max3(m, s[13], s[14]);
+  return fmaxf(m, s[15]);
+}
+
+// Forward.  Work-group = 256 queries of one (segment, head).  K / V tiles of 64 keys go through LDS rings of three
+// tiles (tile i+2 is fetched from memory while tile i is used); within the loop a wave handles 32 keys per step and
+// everything a step needs is requested one step earlier: the scores of step t+1 are computed (MFMA) while the softmax
+// of step t runs (VALU), and the LDS fragments of step t+1 are read while step t computes.  The running stabiliser of
+// a row only moves when a score exceeds it by more than TAU (log2 units).
+template <int ND>
+__global__ __launch_bounds__(256, 1) void attn_fwd_wide(const AttnParams p) {
+  static_assert(ND == 5, "the hand-placed instruction order below is laid out for head_dim 80");
+  using G = Geo<ND>;
+  constexpr int HD = G::HD, NT = 256, BNK = 64, PKW = G::PK, PVW = G::PV;
+  constexpr float TAU = 8.f;
+  __shared__ __attribute__((aligned(16))) bf16_t lds_k[3][BNK * PKW];
+  __shared__ __attribute__((aligned(16))) bf16_t lds_v[3][BNK * PVW];
+  __shared__ __attribute__((aligned(16))) float lds_fix[NT * 4];  // one 16-byte slot per lane (scale_acc, to_acc_regs)
+
+  int seg, h;
+  seg_and_head(p, seg, h);
+  const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
+  const int blk_q0 = blockIdx.x * 256;
+  if (blk_q0 >= L) return;
+  const int l = threadIdx.x & 63, wv = threadIdx.x >> 6, hh = l >> 5, c32 = l & 31, G4 = l >> 4, r = l & 15;
+  const int q0 = blk_q0 + wv * 64;
+
+  const bf16_t* Q = static_cast<const bf16_t*>(p.q) + (int64_t)s0 * p.q_stride + (int64_t)h * HD;
+  const bf16_t* K = static_cast<const bf16_t*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD;
+  const bf16_t* V = static_cast<const bf16_t*>(p.v) + (int64_t)s0 * p.v_stride + (int64_t)h * HD;
+
+  const float c = p.scale * LOG2E;
+  // B operands of the score product (column = query 32*qb + l%32, contraction = head-dim 16*s + 8*(l/32) ..), scaled by
+  // softmax_scale * log2(e) and parked in accumulation registers for the whole kernel
+  u32x4 qf[2][ND];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int qi = q0 + 32 * qb + c32;
+#pragma unroll
+    for (int s = 0; s < ND; ++s)
+      qf[qb][s] = to_acc_regs(scale_frag(load_frag_global(Q + (int64_t)qi * p.q_stride + 16 * s + 8 * hh, qi < L), c), lds_fix + threadIdx.x * 4);
+  }
+  f32x4 o[2][2][ND];
+  f32x16 negm[2];
+  float m_run[2], lsum[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    m_run[qb] = 0.f;
+    lsum[qb] = 0.f;
+    negm[qb] = splat16(0.f);
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+      for (int d = 0; d < ND; ++d) o[qb][hf][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const bf16x2 ones2 = {(bf16_t)1.f, (bf16_t)1.f};
+
+  TileStager<ND, BNK, PKW, NT> sk;
+  TileStager<ND, BNK, PVW, NT> sv;
+  sk.init(p.k_stride);
+  sv.init(p.v_stride);
+  auto rows_from = [&](int k0) { return max(0, min(BNK, L - k0)); };
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    sk.load(K + (int64_t)t * BNK * p.k_stride, rows_from(t * BNK));
+    sv.load(V + (int64_t)t * BNK * p.v_stride, rows_from(t * BNK));
+    sk.store(lds_k[t]);
+    sv.store(lds_v[t]);
+  }
+  __syncthreads();
+
+  struct Frags {
+    bf16x8 kf[ND], vf[ND];
+  };
+  // LDS fragments of one step: K rows krow0.. of tk (scores of the following step), V rows vrow0.. of tv (this step)
+  auto fetch = [&](Frags& f, const bf16_t* tk, int krow0, const bf16_t* tv, int vrow0) {
+#pragma unroll
+    for (int s = 0; s < ND; ++s) f.kf[s] = row_frag32<PKW>(tk, krow0 + c32, s, hh);
+#pragma unroll
+    for (int d = 0; d < ND; ++d) f.vf[d] = tr_block_wide<PVW>(tv, vrow0, d, G4, r);
+  };
+  // Between two steps: masks the keys past the segment end (only the segment's last step can have any), then
+  // moves the stabiliser of rows whose scores outgrew it (rare: taken when any lane of the wave asks for it).
+  auto settle = [&](f32x16 (&sc)[2], float mx0, float mx1, int key0, bool first) {
+    if (key0 + 32 > L) {
+      asm volatile("" ::: "memory");  // keeps this rare block a branch (as selects it would run on every step)
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (key0 + 8 * (i >> 2) + 4 * hh + (i & 3) >= L) sc[qb][i] = -INFINITY;
+      mx0 = max16(sc[0]);
+      mx1 = max16(sc[1]);
+    }
+    if (__builtin_amdgcn_ballot_w64(first || mx0 > TAU || mx1 > TAU) == 0) return;
+    mfma_drain();  // the output accumulators are about to be read by ordinary instructions
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      const float mine = qb == 0 ? mx0 : mx1;
+      const float mfull = fmaxf(mine, other_half(mine));  // over all 32 keys of the step
+      const bool grow = first || mfull > TAU;
+      const float delta = grow ? mfull : 0.f;
+      const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);
+      m_run[qb] += delta;
+      negm[qb] = splat16(-m_run[qb]);
+      lsum[qb] *= alpha;
+      float a0 = alpha, a1 = alpha;
+      swap16f(a0, a1);  // a0: factor of query 32*qb + l%16, a1: of query 32*qb + 16 + l%16
+#pragma unroll
+      for (int d = 0; d < ND; ++d) {
+        scale_acc(o[qb][0][d], a0, lds_fix + threadIdx.x * 4);
+        scale_acc(o[qb][1][d], a1, lds_fix + threadIdx.x * 4);
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sc[qb][i] -= delta;
+    }
+    mfma_drain();
+  };
+  // One 32-key step: softmax numerators of `cur` (scores, ready) -> row sums and O^T += V^T P^T with the V fragments
+  // of `f`, while the scores of the following step are computed from the K fragments of `f` into `nxt` and the
+  // fragments of the following step are read into `fn` (get_next).  The instruction stream alternates matrix and
+  // vector work by hand (a wave is alone on its SIMD): score MFMAs run under the first query block's exp / pack, the
+  // first block's PV MFMAs under the second block's, the second block's PV MFMAs under the row maxima of the new
+  // scores (returned in mx0, mx1).
+  auto step = [&](f32x16 (&cur)[2], f32x16 (&nxt)[2], const Frags& f, auto get_next, float& mx0, float& mx1) {
+    get_next();
+    unsigned w[2][8];
+    auto word = [&](int qb, int j) {
+      w[qb][j] = pack2(__builtin_amdgcn_exp2f(cur[qb][2 * j]), __builtin_amdgcn_exp2f(cur[qb][2 * j + 1]));
+      lsum[qb] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w[qb][j]), ones2, lsum[qb], false);
+    };
+    int done0 = 0, done1 = 0;
+#pragma unroll
+    for (int s = 0; s < ND; ++s) {
+      if (s == 0) {
+        mfma32x32_init(nxt[0], f.kf[0], qf[0][0], negm[0]);
+        mfma32x32_init(nxt[1], f.kf[0], qf[1][0], negm[1]);
+      } else {
+        mfma32x32_acc(nxt[0], f.kf[s], qf[0][s]);
+        mfma32x32_acc(nxt[1], f.kf[s], qf[1][s]);
+      }
+      if (s < 3) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+          if (done0 < 8) word(0, done0++);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          if (done1 < 8) word(1, done1++);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    const BOps p0 = to_b_operands(w[0]);
+    asm volatile("s_nop 1");
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {
+      mfma16_acc(o[0][0][d], f.vf[d], p0.lo);
+      mfma16_acc(o[0][1][d], f.vf[d], p0.hi);
+      if (done1 < 8) word(1, done1++);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    const BOps p1 = to_b_operands(w[1]);
+    asm volatile("s_nop 1");
+    __builtin_amdgcn_sched_barrier(0);
+    float ma = nxt[0][0], mb = nxt[1][0];
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {
+      mfma16_acc(o[1][0][d], f.vf[d], p1.lo);
+      mfma16_acc(o[1][1][d], f.vf[d], p1.hi);
+#pragma unroll
+      for (int i = 1 + 3 * d; i < 1 + 3 * (d + 1); ++i) {
+        ma = fmaxf(ma, nxt[0][i]);
+        mb = fmaxf(mb, nxt[1][i]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    mx0 = ma;
+    mx1 = mb;
+  };
+
+  f32x16 sa[2], sb[2];
+  Frags fa, fb;
+  float mx0, mx1;
+  {  // scores of the first 32 keys, nothing to overlap them with
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+      for (int s = 0; s < ND; ++s) {
+        const bf16x8 kf = row_frag32<PKW>(lds_k[0], c32, s, hh);
+        if (s == 0) mfma32x32_init(sa[qb], kf, qf[qb][0], negm[qb]);
+        else mfma32x32_acc(sa[qb], kf, qf[qb][s]);
+      }
+    mfma_drain();
+    settle(sa, max16(sa[0]), max16(sa[1]), 0, true);
+  }
+  fetch(fa, lds_k[0], 32, lds_v[0], 0);
+  int b0 = 0, b1 = 1, b2 = 2;  // ring slots of this tile, the next one, and the one being filled
+  for (int k0 = 0; k0 < L; k0 += BNK) {
+    sk.load(K + (int64_t)(k0 + 2 * BNK) * p.k_stride, rows_from(k0 + 2 * BNK));
+    sv.load(V + (int64_t)(k0 + 2 * BNK) * p.v_stride, rows_from(k0 + 2 * BNK));
+    // step A: keys k0 .. k0+31 (scores in sa); the scores of keys k0+32 .. k0+63 are computed alongside
+    step(sa, sb, fa, [&] { fetch(fb, lds_k[b1], 0, lds_v[b0], 32); }, mx0, mx1);
+    if (k0 + 32 < L) {
+      settle(sb, mx0, mx1, k0 + 32, false);
+      // step B: keys k0+32 .. k0+63 (scores in sb); the scores of the next tile's first 32 keys alongside
+      step(sb, sa, fb, [&] { fetch(fa, lds_k[b1], 32, lds_v[b1], 0); }, mx0, mx1);
+    }
+    sk.store(lds_k[b2]);  // slot b2 held tile i-1: last read before the barrier that ended the previous iteration
+    sv.store(lds_v[b2]);
+    if (k0 + BNK < L) settle(sa, mx0, mx1, k0 + BNK, false);
+    __syncthreads();
+    const int t = b0;
+    b0 = b1;
+    b1 = b2;
+    b2 = t;
+  }
+  mfma_drain();
+
+  bf16_t* O = static_cast<bf16_t*>(p.out) + (int64_t)s0 * p.o_stride + (int64_t)h * HD;
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const float lt = lsum[qb] + other_half(lsum[qb]);
+    float i0 = 1.f / lt, i1 = i0;
+    swap16f(i0, i1);
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const int qi = q0 + 32 * qb + 16 * hf + r;
+      if (qi < L) {
+        const float inv = hf == 0 ? i0 : i1;
+#pragma unroll
+        for (int d = 0; d < ND; ++d) {
+          bf16x4 ov;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) ov[i] = (bf16_t)(o[qb][hf][d][i] * inv);
+          *reinterpret_cast<bf16x4*>(O + (int64_t)qi * p.o_stride + 16 * d + 4 * G4) = ov;
+        }
+      }
+    }
+    const int qi = q0 + 32 * qb + c32;
+    if (hh == 0 && qi < L) p.lse[(int64_t)h * p.total + s0 + qi] = (m_run[qb] + __builtin_amdgcn_logf(lt)) * LN2;
+  }
+}
+
 // delta[h, s] = sum_d O[s,h,d] * dO[s,h,d].  One lane per (row, head), 16-byte loads; neighbouring lanes take
 // neighbouring heads of the same row, so a wave sweeps contiguous memory.
 template <typename T>
@@ -728,6 +1107,318 @@ __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dkdv_mfma(const AttnPara
         }
         *reinterpret_cast<bf16x4*>(DK + (int64_t)ki * p.dk_stride + 16 * d + 4 * g) = a;
         *reinterpret_cast<bf16x4*>(DV + (int64_t)ki * p.dv_stride + 16 * d + 4 * g) = b;
+      }
+    }
+  }
+}
+
+// ================================================================================================
+// LDS tile layout of the wide backward kernels: 32 rows of 256 bytes (16 slots of 16 bytes, 10 of them used at head_dim
+// 80); chunk c of row r lives in slot c ^ xs(r), xs(r) = 2*(r & 3) + ((r >> 2) & 1).  Eight consecutive rows put one
+// chunk index into eight different slots (16-byte row-fragment reads), four consecutive rows put one pair of chunks
+// into four different 32-byte windows (transposing reads): neither pattern has bank conflicts.  The tile is filled by
+// global_load_lds_dwordx4 (16 bytes per lane straight into LDS at M0 + 16 * lane, no staging registers): lane i of
+// instruction j fills slot 64*j + i, i.e. it fetches chunk (i & 15) ^ xs(row) of row 4*j + i/16.
+constexpr int XS_PITCH = 128;                 // elements per LDS row
+constexpr int XS_TILE = 32 * XS_PITCH;        // elements per 32-row tile (8 KiB)
+__device__ __forceinline__ int xs(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
+__device__ __forceinline__ bf16x8 xs_row_frag(const bf16_t* tile, int row, int s, int h) {
+  return *reinterpret_cast<const bf16x8*>(tile + row * XS_PITCH + (((2 * s + h) ^ xs(row)) << 3));
+}
+// transposed A operand (see tr_block_wide) of head-dim block d from rows base(G) + (r >> 2) and + 8
+__device__ __forceinline__ bf16x8 xs_tr_block(const bf16_t* tile, int d, int G, int r) {
+  const int row = 16 * (G & 1) + 4 * (G >> 1) + (r >> 2);
+  const bf16_t* a = tile + row * XS_PITCH + (((2 * d + ((r & 3) >> 1)) ^ xs(row)) << 3) + 4 * (r & 1);
+  return tr_pair(a, a + 8 * XS_PITCH);  // xs(row + 8) == xs(row)
+}
+// wave-uniform values as scalars (the compiler cannot prove uniformity of values derived from the wave index)
+__device__ __forceinline__ unsigned uniform_u32(unsigned x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ const void* uniform_ptr(const void* q) {
+  const uint64_t v = (uint64_t)(uintptr_t)q;
+  const uint64_t u = (uint64_t)uniform_u32((unsigned)v) | ((uint64_t)uniform_u32((unsigned)(v >> 32)) << 32);
+  return (const void*)(uintptr_t)u;
+}
+// lds_addr and base must be wave-uniform (scalar registers)
+__device__ __forceinline__ void lds_direct_16(unsigned lds_addr, unsigned voff, const void* base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+__device__ __forceinline__ void lds_direct_4(unsigned lds_addr, unsigned voff, const void* base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// q_scaled[s, h, :] = bf16(q[s, h, :] * c) for the wide backward kernels (the forward rounds Q * scale * log2(e) to
+// bf16 the same way, so the recomputed probabilities match the forward's), and the row statistics in the form the
+// MFMA accumulators are initialised with: nlse2 = - lse * log2(e), ndelta = - delta.
+__global__ __launch_bounds__(256) void attn_bwd_prepare_kernel(const bf16_t* __restrict__ q, int64_t q_stride, bf16_t* __restrict__ qs,
+                                                               int64_t qs_stride, int64_t total, int cols, float c,
+                                                               const float* __restrict__ lse, const float* __restrict__ delta,
+                                                               float* __restrict__ nlse2, float* __restrict__ ndelta, int64_t nstat) {
+  const int cpr = cols / 8;
+  const int64_t nchunk = total * cpr;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nchunk; i += (int64_t)gridDim.x * 256) {
+    const int64_t row = i / cpr;
+    const int ch = (int)(i % cpr);
+    bf16x8 v = *reinterpret_cast<const bf16x8*>(q + row * q_stride + ch * 8);
+    *reinterpret_cast<bf16x8*>(qs + row * qs_stride + ch * 8) = scale_frag(v, c);
+  }
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nstat; i += (int64_t)gridDim.x * 256) {
+    nlse2[i] = -lse[i] * LOG2E;
+    ndelta[i] = -delta[i];
+  }
+}
+
+// ================================================================================================
+// dK, dV for long segments, "wide" form: a wave owns 64 keys (two groups of 32), four waves = 256 keys per work-group,
+// one work-group per CU.  K / V fragments of the wave's keys and the 2 x 80 accumulators live in accumulation
+// registers; pre-scaled Q / dO tiles of 32 queries and their statistics stream through an LDS ring of four tiles,
+// written by direct global -> LDS loads three tiles ahead.  Per tile and key group:
+//   S = Q K^T - lse2, dP = dO V^T - delta   (v_mfma_f32_32x32x16_bf16, head_dim contracted exactly; the first MFMA of
+//                                            a chain takes the tile of "- statistic" values as its accumulator input)
+//   P = exp2(S), dS = P * dP                 (vector ALU), packed to bf16 and turned into B operands by lane swaps
+//   dV^T += dO^T P, dK^T += Q^T dS           (v_mfma_f32_16x16x32_bf16, transposed left factors read from LDS)
+// A wave is alone on its SIMD, so matrix and vector instructions are interleaved by hand: the second key group's
+// score MFMAs run under the first group's exp / pack, the first group's dV / dK MFMAs under the second group's.
+template <int ND>
+__global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p) {
+  static_assert(ND == 5, "the hand-placed instruction order below is laid out for head_dim 80");
+  using G = Geo<ND>;
+  constexpr int HD = G::HD, BQ = 32, NT = 256, RING = 4;
+  __shared__ __attribute__((aligned(1024))) bf16_t lds_q[RING][XS_TILE];
+  __shared__ __attribute__((aligned(1024))) bf16_t lds_do[RING][XS_TILE];
+  __shared__ __attribute__((aligned(256))) float lds_nlse[RING][64];  // - lse * log2(e) per query of the tile (32 used)
+  __shared__ __attribute__((aligned(256))) float lds_ndel[RING][64];  // - delta
+  __shared__ __attribute__((aligned(16))) float lds_fix[NT * 4];
+
+  int seg, h;
+  seg_and_head(p, seg, h);
+  const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
+  const int blk_k0 = blockIdx.x * 256;
+  if (blk_k0 >= L) return;
+  const int l = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), hh = l >> 5, c32 = l & 31, G4 = l >> 4, r = l & 15;
+  const int key0 = blk_k0 + wv * 64;
+
+  const bf16_t* QS = static_cast<const bf16_t*>(p.q_scaled) + (int64_t)s0 * p.qs_stride + (int64_t)h * HD;
+  const bf16_t* K = static_cast<const bf16_t*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD;
+  const bf16_t* V = static_cast<const bf16_t*>(p.v) + (int64_t)s0 * p.v_stride + (int64_t)h * HD;
+  const bf16_t* DO = static_cast<const bf16_t*>(p.d_o) + (int64_t)s0 * p.do_stride + (int64_t)h * HD;
+  const float* NLSE = p.nlse2 + (int64_t)h * p.total + s0;
+  const float* NDEL = p.ndelta + (int64_t)h * p.total + s0;
+
+  // B operands of the score products (column = key 32*kg + l%32, contraction = head-dim 16*s + 8*(l/32) ..)
+  u32x4 kf[2][ND], vf[2][ND];
+#pragma unroll
+  for (int kg = 0; kg < 2; ++kg) {
+    const int ki = key0 + 32 * kg + c32;
+#pragma unroll
+    for (int s = 0; s < ND; ++s) {
+      kf[kg][s] = to_acc_regs(load_frag_global(K + (int64_t)ki * p.k_stride + 16 * s + 8 * hh, ki < L), lds_fix + threadIdx.x * 4);
+      vf[kg][s] = to_acc_regs(load_frag_global(V + (int64_t)ki * p.v_stride + 16 * s + 8 * hh, ki < L), lds_fix + threadIdx.x * 4);
+    }
+  }
+  f32x4 dk[4][ND], dv[4][ND];  // [16-key block][16-wide head-dim block]: lane = key l%16, registers = head-dim 4*(l/16) + i
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {
+      dk[kb][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+      dv[kb][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+  // Direct global -> LDS loads: per tile and tensor eight 1 KiB instructions, two of them this wave's; wave 0 and 1 also
+  // fetch one array of statistics each.  Rows past the segment end are read from the segment's last row (they stay
+  // finite and meet a probability of exactly zero: their statistics are overwritten before use).
+  int trow[2], tchunk[2];
+  unsigned voff_q[2], voff_do[2];  // byte offsets of this lane's chunks from the tile's first row (tiles without a tail)
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int slot = 64 * (2 * wv + j) + l;
+    trow[j] = slot >> 4;
+    tchunk[j] = min(((slot & 15) ^ xs(trow[j])), 2 * ND - 1);  // padding slots re-fetch the last chunk
+    voff_q[j] = (unsigned)(trow[j] * (int)p.qs_stride * 2 + tchunk[j] * 16);
+    voff_do[j] = (unsigned)(trow[j] * (int)p.do_stride * 2 + tchunk[j] * 16);
+  }
+  const unsigned lds_q0 = (unsigned)(uintptr_t)&lds_q[0][0], lds_do0 = (unsigned)(uintptr_t)&lds_do[0][0];
+  const unsigned lds_nl0 = (unsigned)(uintptr_t)&lds_nlse[0][0], lds_nd0 = (unsigned)(uintptr_t)&lds_ndel[0][0];
+  auto request_tile = [&](int qs, int slot) {  // 5 (waves 0, 1) or 4 load instructions
+    if (qs >= L) return;
+    const int last = L - 1 - qs;  // last valid row of the tile (>= 0)
+    const bool tail = last < BQ - 1;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      unsigned vq = voff_q[j], vd = voff_do[j];
+      if (tail) {
+        const int row = min(trow[j], last);
+        vq = (unsigned)(row * (int)p.qs_stride * 2 + tchunk[j] * 16);
+        vd = (unsigned)(row * (int)p.do_stride * 2 + tchunk[j] * 16);
+      }
+      lds_direct_16(lds_q0 + slot * (XS_TILE * 2) + (2 * wv + j) * 1024, vq, QS + (int64_t)qs * p.qs_stride);
+      lds_direct_16(lds_do0 + slot * (XS_TILE * 2) + (2 * wv + j) * 1024, vd, DO + (int64_t)qs * p.do_stride);
+    }
+    if (wv < 2) lds_direct_4((wv == 0 ? lds_nl0 : lds_nd0) + slot * 256, (unsigned)(min(l, last) * 4), (wv == 0 ? NLSE : NDEL) + qs);
+  };
+  // statistics of rows past the segment end: probability zero, no contribution
+  auto fix_tail = [&](int qs, int slot) {
+    if (qs < L && qs + BQ > L && threadIdx.x < BQ && qs + (int)threadIdx.x >= L) {
+      lds_nlse[slot][threadIdx.x] = -1e30f;
+      lds_ndel[slot][threadIdx.x] = 0.f;
+    }
+  };
+  request_tile(0, 0);
+  request_tile(BQ, 1);
+  request_tile(2 * BQ, 2);
+  wait_vmcnt<0>();
+  fix_tail(0, 0);
+  fix_tail(BQ, 1);
+  fix_tail(2 * BQ, 2);
+  __syncthreads();
+
+  bf16x8 qa[ND], da[ND];  // A operands of the score products: row = query l%32 of the tile
+  f32x16 nl, nd;          // - lse2 and - delta of the tile's queries in accumulator layout (register i: query 8*(i/4) + 4*(l/32) + i%4)
+  f32x16 sc[2], dp[2];    // per key group: S - lse2 and dP - delta, lane = key l%32
+  auto fetch_rows = [&](int slot) {
+#pragma unroll
+    for (int s = 0; s < ND; ++s) {
+      qa[s] = xs_row_frag(lds_q[slot], c32, s, hh);
+      da[s] = xs_row_frag(lds_do[slot], c32, s, hh);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(&lds_nlse[slot][8 * j + 4 * hh]);
+      const f32x4 b = *reinterpret_cast<const f32x4*>(&lds_ndel[slot][8 * j + 4 * hh]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        nl[4 * j + i] = a[i];
+        nd[4 * j + i] = b[i];
+      }
+    }
+  };
+  fetch_rows(0);
+
+#ifdef MVIT_STAMP
+  long long stamp_acc[6] = {0, 0, 0, 0, 0, 0};
+  long long t_prev = __builtin_readcyclecounter();
+#define STAMP(i) { __builtin_amdgcn_sched_barrier(0); long long t_now = __builtin_readcyclecounter(); stamp_acc[i] += t_now - t_prev; t_prev = t_now; __builtin_amdgcn_sched_barrier(0); }
+#else
+#define STAMP(i)
+#endif
+  int it = 0;
+  for (int qs = 0; qs < L; qs += BQ, ++it) {
+    const int b0 = it & 3, b1 = (it + 1) & 3, b3 = (it + 3) & 3;
+    // tile it+3 is requested into the slot that tile it-1 left (every wave is past the barrier that ended iteration it-1)
+    request_tile(qs + 3 * BQ, b3);
+    STAMP(5)
+    // ---- phase 1: score products of key group 0; the transposed left factors that phase 3 needs are read from LDS
+    // between the MFMAs
+    bf16x8 qt[ND], dt_[ND];
+#pragma unroll
+    for (int s = 0; s < ND; ++s) {
+      if (s == 0) {
+        mfma32x32_init(sc[0], qa[0], kf[0][0], nl);
+        mfma32x32_init(dp[0], da[0], vf[0][0], nd);
+      } else {
+        mfma32x32_acc(sc[0], qa[s], kf[0][s]);
+        mfma32x32_acc(dp[0], da[s], vf[0][s]);
+      }
+      qt[s] = xs_tr_block(lds_q[b0], s, G4, r);
+      dt_[s] = xs_tr_block(lds_do[b0], s, G4, r);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    STAMP(0)
+    // ---- phase 2: score products of key group 1 under the vector work of group 0
+    unsigned pw[8], dw[8];
+    auto words = [&](int j) {
+      const float e0 = __builtin_amdgcn_exp2f(sc[0][2 * j]), e1 = __builtin_amdgcn_exp2f(sc[0][2 * j + 1]);
+      pw[j] = pack2(e0, e1);
+      dw[j] = pack2(e0 * dp[0][2 * j], e1 * dp[0][2 * j + 1]);
+    };
+    int done = 0;
+#pragma unroll
+    for (int s = 0; s < ND; ++s) {
+      if (s == 0) {
+        mfma32x32_init(sc[1], qa[0], kf[1][0], nl);
+        mfma32x32_init(dp[1], da[0], vf[1][0], nd);
+      } else {
+        mfma32x32_acc(sc[1], qa[s], kf[1][s]);
+        mfma32x32_acc(dp[1], da[s], vf[1][s]);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        if (done < 8) words(done++);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    BOps pb = to_b_operands(pw), db = to_b_operands(dw);
+    asm volatile("s_nop 1");
+    __builtin_amdgcn_sched_barrier(0);
+    STAMP(1)
+    // ---- phase 3: dV / dK of key group 0 under the vector work of group 1
+    unsigned pw1[8], dw1[8];
+    auto words1 = [&](int j) {
+      const float e0 = __builtin_amdgcn_exp2f(sc[1][2 * j]), e1 = __builtin_amdgcn_exp2f(sc[1][2 * j + 1]);
+      pw1[j] = pack2(e0, e1);
+      dw1[j] = pack2(e0 * dp[1][2 * j], e1 * dp[1][2 * j + 1]);
+    };
+    done = 0;
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {
+      dv[0][d] = mfma32(dt_[d], pb.lo, dv[0][d]);
+      dk[0][d] = mfma32(qt[d], db.lo, dk[0][d]);
+      dv[1][d] = mfma32(dt_[d], pb.hi, dv[1][d]);
+      dk[1][d] = mfma32(qt[d], db.hi, dk[1][d]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        if (done < 8) words1(done++);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    BOps pb1 = to_b_operands(pw1), db1 = to_b_operands(dw1);
+    asm volatile("s_nop 1");
+    __builtin_amdgcn_sched_barrier(0);
+    STAMP(2)
+    // ---- phase 4: dV / dK of key group 1 under the fragment reads of the next tile; the barrier is waited for while
+    // these MFMAs drain
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {
+      dv[2][d] = mfma32(dt_[d], pb1.lo, dv[2][d]);
+      dk[2][d] = mfma32(qt[d], db1.lo, dk[2][d]);
+      dv[3][d] = mfma32(dt_[d], pb1.hi, dv[3][d]);
+      dk[3][d] = mfma32(qt[d], db1.hi, dk[3][d]);
+    }
+    fetch_rows(b1);
+    STAMP(3)
+    // tile it+2 (requested in iteration it-1) must have landed before any wave reads it in the next iteration; the
+    // loads requested in this iteration (at most five) may stay in flight
+    if (qs + 3 * BQ < L) wait_vmcnt<5>();
+    else wait_vmcnt<0>();
+    fix_tail(qs + 2 * BQ, (it + 2) & 3);
+    __syncthreads();
+    STAMP(4)
+  }
+
+#ifdef MVIT_STAMP
+  if (blockIdx.x == 3 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 64) {
+    printf("stamps (ticks, %d iterations): ph1 %lld ph2 %lld ph3 %lld ph4 %lld barrier %lld store %lld\n", (L + BQ - 1) / BQ,
+           stamp_acc[0], stamp_acc[1], stamp_acc[2], stamp_acc[3], stamp_acc[4], stamp_acc[5]);
+  }
+#endif
+  bf16_t* DK = static_cast<bf16_t*>(p.dk) + (int64_t)s0 * p.dk_stride + (int64_t)h * HD;
+  bf16_t* DV = static_cast<bf16_t*>(p.dv) + (int64_t)s0 * p.dv_stride + (int64_t)h * HD;
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) {
+    const int ki = key0 + kb * 16 + r;
+    if (ki < L) {
+#pragma unroll
+      for (int d = 0; d < ND; ++d) {
+        bf16x4 a, b;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          a[i] = (bf16_t)(dk[kb][d][i] * LN2);  // dS^T (Q scale log2e) / log2e
+          b[i] = (bf16_t)dv[kb][d][i];
+        }
+        *reinterpret_cast<bf16x4*>(DK + (int64_t)ki * p.dk_stride + 16 * d + 4 * G4) = a;
+        *reinterpret_cast<bf16x4*>(DV + (int64_t)ki * p.dv_stride + 16 * d + 4 * G4) = b;
       }
     }
   }
@@ -1252,6 +1943,7 @@ __global__ __launch_bounds__(64) void attn_bwd_dkdv_f32(const AttnParams p) {
 }
 
 // ------------------------------------------------------------------------------------------------
+constexpr int WIDE_MIN_SEQLEN = 512;  // from here on the 64-rows-per-wave kernels fill their work-groups well enough
 inline int pick_waves(int max_seqlen) { return max_seqlen <= 64 ? 1 : (max_seqlen <= 128 ? 2 : 4); }
 
 template <int ND>
@@ -1265,6 +1957,12 @@ int launch_fwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
     if constexpr (ND <= 5) hipLaunchKernelGGL((attn_fwd_mfma<ND, 2, 64, false, 2, 4>), grid, 128, 0, s, pw);
   } else if (nw == 1) hipLaunchKernelGGL((attn_fwd_mfma<ND, 1, 64, false>), grid, 64, 0, s, p);
   else if (nw == 2) hipLaunchKernelGGL((attn_fwd_mfma<ND, 2, 64, false>), grid, 128, 0, s, p);
+  else if (ND == 5 && max_seqlen >= WIDE_MIN_SEQLEN && false) {
+    AttnParams pl = p;
+    pl.seg_major = 1;
+    dim3 gl((unsigned)((max_seqlen + 255) / 256), (unsigned)p.nheads, (unsigned)n_seg);
+    if constexpr (ND == 5) hipLaunchKernelGGL((attn_fwd_wide<ND>), gl, 256, 0, s, pl);
+  }
   else if constexpr (ND <= 5) {
     // long segments: 8 waves x 32 queries, <= 128 registers, so that four waves share a SIMD and cover each
     // other's MFMA -> softmax -> MFMA dependency stalls
@@ -1279,6 +1977,7 @@ int launch_fwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
   MVIT_CHECK_LAUNCH("attn_fwd");
   return MVIT_OK;
 }
+using G5 = Geo<5>;
 template <int ND>
 int launch_bwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t s) {
   // short segments (windows): one work-group does the whole backward of a (segment, head); long ones: 8 waves x 32 rows
@@ -1302,7 +2001,25 @@ int launch_bwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
     AttnParams pl = p;
     pl.seg_major = 1;  // as in the forward: segment-major launch order
     dim3 gl = pl.seg_major ? dim3(grid.x, grid.z, grid.y) : grid;
-    hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 8, 2>), gl, 512, 0, s, pl);
+    if (ND == 5 && max_seqlen >= WIDE_MIN_SEQLEN) {
+      if constexpr (ND == 5) {
+        // the dq buffer holds the pre-scaled queries until the dQ kernel overwrites it with the result
+        const int64_t nstat = (int64_t)p.nheads * p.total;
+        pl.q_scaled = p.dq;
+        pl.qs_stride = p.dq_stride;
+        pl.nlse2 = p.delta + nstat;
+        pl.ndelta = p.delta + 2 * nstat;
+        const int cols = p.nheads * G5::HD;
+        const int64_t nchunk = p.total * (cols / 8);
+        const unsigned pgrid = (unsigned)std::min<int64_t>(8192, (std::max(nchunk, nstat) + 255) / 256);
+        hipLaunchKernelGGL(attn_bwd_prepare_kernel, dim3(pgrid), 256, 0, s, static_cast<const bf16_t*>(p.q), p.q_stride,
+                           static_cast<bf16_t*>(p.dq), p.dq_stride, p.total, cols, p.scale * LOG2E, (const float*)p.lse,
+                           (const float*)p.delta, p.delta + nstat, p.delta + 2 * nstat, nstat);
+        hipLaunchKernelGGL((attn_bwd_dkdv_wide<ND>), gl, 256, 0, s, pl);
+      }
+    } else {
+      hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 8, 2>), gl, 512, 0, s, pl);
+    }
     hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 8, 2>), gl, 512, 0, s, pl);
   }
   MVIT_CHECK_LAUNCH("attn_bwd");

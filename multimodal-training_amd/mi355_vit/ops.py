@@ -443,7 +443,7 @@ def attn_bwd(q, k, v, o, d_o, lse, cu_seqlens, max_seqlen, nheads, head_dim, sca
             raise ValueError("attn_bwd: row count / dtype mismatch")
     if tuple(lse.shape) != (nheads, S) or lse.dtype != torch.float32 or not lse.is_contiguous():
         raise ValueError("attn_bwd: lse must be contiguous fp32 [nheads, S]")
-    delta = torch.empty(nheads, S, dtype=torch.float32, device=q.device)
+    delta = torch.empty(3, nheads, S, dtype=torch.float32, device=q.device)  # workspace: delta, -lse*log2(e), -delta
     st = _stream(q)
     strides = tuple(_attn_view(t, nheads, head_dim, nm) for t, nm in ((q, "q"), (k, "k"), (v, "v"), (o, "o"), (d_o, "do"), (dq, "dq"), (dk, "dk"), (dv, "dv")))
     rc = _launch("attn_bwd", {"cu": cu_seqlens, "max_seqlen": max_seqlen, "nheads": nheads, "head_dim": head_dim}, lambda: _lib.load().mvit_attn_bwd(
