@@ -1425,6 +1425,224 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
 }
 
 // ================================================================================================
+// dQ for long segments, "wide" form: a wave owns 64 queries (two blocks of 32), four waves = 256 queries per
+// work-group, one work-group per CU.  Pre-scaled Q and dO fragments of the wave's queries, and the 80 accumulators,
+// live in accumulation registers; K / V tiles of 32 keys stream through an LDS ring of four tiles (direct
+// global -> LDS loads, three tiles ahead).  Per tile and query block:
+//   S^T = K Q^T - lse2, dP^T = V dO^T - delta   (v_mfma_f32_32x32x16_bf16; lane = query, so the statistics are per-lane
+//                                                constants kept as ready-made accumulator input tiles)
+//   dS^T = exp2(S^T) * dP^T                      (vector ALU), packed to bf16, lane swaps
+//   dQ^T += K^T dS^T                             (v_mfma_f32_16x16x32_bf16, K^T read from LDS with the transposing load)
+template <int ND>
+__global__ __launch_bounds__(256, 1) void attn_bwd_dq_wide(const AttnParams p) {
+  static_assert(ND == 5, "the hand-placed instruction order below is laid out for head_dim 80");
+  using G = Geo<ND>;
+  constexpr int HD = G::HD, BK = 32, NT = 256, RING = 4;
+  __shared__ __attribute__((aligned(1024))) bf16_t lds_k[RING][XS_TILE];
+  __shared__ __attribute__((aligned(1024))) bf16_t lds_v[RING][XS_TILE];
+  __shared__ __attribute__((aligned(16))) float lds_fix[NT * 4];
+
+  int seg, h;
+  seg_and_head(p, seg, h);
+  const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
+  const int blk_q0 = blockIdx.x * 256;
+  if (blk_q0 >= L) return;
+  const int l = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), hh = l >> 5, c32 = l & 31, G4 = l >> 4, r = l & 15;
+  const int q0 = blk_q0 + wv * 64;
+
+  const bf16_t* QS = static_cast<const bf16_t*>(p.q_scaled) + (int64_t)s0 * p.qs_stride + (int64_t)h * HD;
+  const bf16_t* K = static_cast<const bf16_t*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD;
+  const bf16_t* V = static_cast<const bf16_t*>(p.v) + (int64_t)s0 * p.v_stride + (int64_t)h * HD;
+  const bf16_t* DO = static_cast<const bf16_t*>(p.d_o) + (int64_t)s0 * p.do_stride + (int64_t)h * HD;
+  const float* NLSE = p.nlse2 + (int64_t)h * p.total + s0;
+  const float* NDEL = p.ndelta + (int64_t)h * p.total + s0;
+
+  // B operands of the score products (column = query 32*qb + l%32, contraction = head-dim 16*s + 8*(l/32) ..) and the
+  // accumulator input tiles holding the query's - lse2 / - delta in all sixteen registers
+  u32x4 qf[2][ND], dof[2][ND];
+  f32x16 nl[2], nd[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int qi = q0 + 32 * qb + c32;
+    const bool ok = qi < L;
+#pragma unroll
+    for (int s = 0; s < ND; ++s) {
+      qf[qb][s] = to_acc_regs(load_frag_global(QS + (int64_t)qi * p.qs_stride + 16 * s + 8 * hh, ok), lds_fix + threadIdx.x * 4);
+      dof[qb][s] = to_acc_regs(load_frag_global(DO + (int64_t)qi * p.do_stride + 16 * s + 8 * hh, ok), lds_fix + threadIdx.x * 4);
+    }
+    nl[qb] = splat16(ok ? NLSE[qi] : -1e30f);  // hugely negative => p = 0 for queries past the end
+    nd[qb] = splat16(ok ? NDEL[qi] : 0.f);
+  }
+  f32x4 dq[2][2][ND];  // [query block][half][head-dim block]: lane = query l%16 of the half, registers = head-dim 4*(l/16) + i
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+      for (int d = 0; d < ND; ++d) dq[qb][hf][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // direct global -> LDS loads of the K / V tiles (see attn_bwd_dkdv_wide); rows past the segment end repeat its last row
+  int trow[2], tchunk[2];
+  unsigned voff_k[2], voff_v[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int slot = 64 * (2 * wv + j) + l;
+    trow[j] = slot >> 4;
+    tchunk[j] = min(((slot & 15) ^ xs(trow[j])), 2 * ND - 1);
+    voff_k[j] = (unsigned)(trow[j] * (int)p.k_stride * 2 + tchunk[j] * 16);
+    voff_v[j] = (unsigned)(trow[j] * (int)p.v_stride * 2 + tchunk[j] * 16);
+  }
+  const unsigned lds_k0 = (unsigned)(uintptr_t)&lds_k[0][0], lds_v0 = (unsigned)(uintptr_t)&lds_v[0][0];
+  auto request_tile = [&](int k0, int slot) {  // 4 load instructions
+    if (k0 >= L) return;
+    const int last = L - 1 - k0;
+    const bool tail = last < BK - 1;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      unsigned vk = voff_k[j], vv = voff_v[j];
+      if (tail) {
+        const int row = min(trow[j], last);
+        vk = (unsigned)(row * (int)p.k_stride * 2 + tchunk[j] * 16);
+        vv = (unsigned)(row * (int)p.v_stride * 2 + tchunk[j] * 16);
+      }
+      lds_direct_16(lds_k0 + slot * (XS_TILE * 2) + (2 * wv + j) * 1024, vk, K + (int64_t)k0 * p.k_stride);
+      lds_direct_16(lds_v0 + slot * (XS_TILE * 2) + (2 * wv + j) * 1024, vv, V + (int64_t)k0 * p.v_stride);
+    }
+  };
+  request_tile(0, 0);
+  request_tile(BK, 1);
+  request_tile(2 * BK, 2);
+  wait_vmcnt<0>();
+  __syncthreads();
+
+  bf16x8 ka[ND], va[ND];  // A operands of the score products: row = key l%32 of the tile
+  auto fetch_rows = [&](int slot) {
+#pragma unroll
+    for (int s = 0; s < ND; ++s) {
+      ka[s] = xs_row_frag(lds_k[slot], c32, s, hh);
+      va[s] = xs_row_frag(lds_v[slot], c32, s, hh);
+    }
+  };
+  fetch_rows(0);
+
+  f32x16 sc[2], dp[2];  // per query block: S^T - lse2 and dP^T - delta, lane = query l%32, register i = key 8*(i/4) + 4*(l/32) + i%4
+#ifdef MVIT_STAMP
+  long long stamp_acc[6] = {0, 0, 0, 0, 0, 0};
+  long long t_prev = __builtin_readcyclecounter();
+#endif
+  int it = 0;
+  for (int k0 = 0; k0 < L; k0 += BK, ++it) {
+    const int b0 = it & 3, b1 = (it + 1) & 3, b3 = (it + 3) & 3;
+    request_tile(k0 + 3 * BK, b3);
+    STAMP(5)
+    const int valid = L - k0;  // keys of this tile inside the segment (>= 1)
+    // ---- phase 1: score products of query block 0; K^T fragments for the dQ products are read between the MFMAs
+    bf16x8 kt[ND];
+#pragma unroll
+    for (int s = 0; s < ND; ++s) {
+      if (s == 0) {
+        mfma32x32_init(sc[0], ka[0], qf[0][0], nl[0]);
+        mfma32x32_init(dp[0], va[0], dof[0][0], nd[0]);
+      } else {
+        mfma32x32_acc(sc[0], ka[s], qf[0][s]);
+        mfma32x32_acc(dp[0], va[s], dof[0][s]);
+      }
+      kt[s] = xs_tr_block(lds_k[b0], s, G4, r);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    STAMP(0)
+    // ---- phase 2: score products of query block 1 under the vector work of block 0
+    unsigned dw[2][8];
+    auto word = [&](int qb, int j) {
+      const float x0 = __builtin_amdgcn_exp2f(sc[qb][2 * j]) * dp[qb][2 * j], x1 = __builtin_amdgcn_exp2f(sc[qb][2 * j + 1]) * dp[qb][2 * j + 1];
+      dw[qb][j] = pack2(x0, x1);
+    };
+    // keys past the segment end (last tile only) contribute nothing: their dP is zeroed before it is used
+    auto mask_tail = [&](int qb) {
+      if (valid < BK) {
+        asm volatile("" ::: "memory");  // keeps this rare block a branch
+        mfma_drain();
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (8 * (i >> 2) + 4 * hh + (i & 3) >= valid) dp[qb][i] = 0.f;
+      }
+    };
+    mask_tail(0);
+    int done = 0;
+#pragma unroll
+    for (int s = 0; s < ND; ++s) {
+      if (s == 0) {
+        mfma32x32_init(sc[1], ka[0], qf[1][0], nl[1]);
+        mfma32x32_init(dp[1], va[0], dof[1][0], nd[1]);
+      } else {
+        mfma32x32_acc(sc[1], ka[s], qf[1][s]);
+        mfma32x32_acc(dp[1], va[s], dof[1][s]);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        if (done < 8) word(0, done++);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    const BOps d0 = to_b_operands(dw[0]);
+    asm volatile("s_nop 1");
+    __builtin_amdgcn_sched_barrier(0);
+    STAMP(1)
+    // ---- phase 3: dQ of query block 0 under the vector work of block 1
+    mask_tail(1);
+    done = 0;
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {
+      dq[0][0][d] = mfma32(kt[d], d0.lo, dq[0][0][d]);
+      dq[0][1][d] = mfma32(kt[d], d0.hi, dq[0][1][d]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        if (done < 8) word(1, done++);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    const BOps d1 = to_b_operands(dw[1]);
+    asm volatile("s_nop 1");
+    __builtin_amdgcn_sched_barrier(0);
+    STAMP(2)
+    // ---- phase 4: dQ of query block 1 under the fragment reads of the next tile
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {
+      dq[1][0][d] = mfma32(kt[d], d1.lo, dq[1][0][d]);
+      dq[1][1][d] = mfma32(kt[d], d1.hi, dq[1][1][d]);
+    }
+    fetch_rows(b1);
+    STAMP(3)
+    // tile it+2 (requested in iteration it-1) must have landed before any wave reads it in the next iteration
+    if (k0 + 3 * BK < L) wait_vmcnt<4>();
+    else wait_vmcnt<0>();
+    __syncthreads();
+    STAMP(4)
+  }
+#ifdef MVIT_STAMP
+  if (blockIdx.x == 3 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 64) {
+    printf("dq stamps (ticks, %d iterations): ph1 %lld ph2 %lld ph3 %lld ph4 %lld barrier %lld request %lld\n", (L + BK - 1) / BK,
+           stamp_acc[0], stamp_acc[1], stamp_acc[2], stamp_acc[3], stamp_acc[4], stamp_acc[5]);
+  }
+#endif
+
+  bf16_t* DQ = static_cast<bf16_t*>(p.dq) + (int64_t)s0 * p.dq_stride + (int64_t)h * HD;
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const int qi = q0 + 32 * qb + 16 * hf + r;
+      if (qi < L) {
+#pragma unroll
+        for (int d = 0; d < ND; ++d) {
+          bf16x4 a;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) a[i] = (bf16_t)(dq[qb][hf][d][i] * p.scale);
+          *reinterpret_cast<bf16x4*>(DQ + (int64_t)qi * p.dq_stride + 16 * d + 4 * G4) = a;
+        }
+      }
+    }
+}
+
+// ================================================================================================
 // dQ.  Block = 64*NWAVES queries of one (segment, head); 32 keys per iteration, K / V tiles double buffered.
 template <int ND, int NWAVES, int RB>
 __global__ __launch_bounds__(64 * NWAVES) void attn_bwd_dq_mfma(const AttnParams p) {
@@ -2016,11 +2234,12 @@ int launch_bwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
                            static_cast<bf16_t*>(p.dq), p.dq_stride, p.total, cols, p.scale * LOG2E, (const float*)p.lse,
                            (const float*)p.delta, p.delta + nstat, p.delta + 2 * nstat, nstat);
         hipLaunchKernelGGL((attn_bwd_dkdv_wide<ND>), gl, 256, 0, s, pl);
+        hipLaunchKernelGGL((attn_bwd_dq_wide<ND>), gl, 256, 0, s, pl);
       }
     } else {
       hipLaunchKernelGGL((attn_bwd_dkdv_mfma<ND, 8, 2>), gl, 512, 0, s, pl);
+      hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 8, 2>), gl, 512, 0, s, pl);
     }
-    hipLaunchKernelGGL((attn_bwd_dq_mfma<ND, 8, 2>), gl, 512, 0, s, pl);
   }
   MVIT_CHECK_LAUNCH("attn_bwd");
   return MVIT_OK;
