@@ -1297,6 +1297,20 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
     }
   };
   fetch_rows(0);
+  // the same reads in five parts (one per head-dim step), to sit between MFMAs
+  auto fetch_rows_part = [&](int slot, int s) {
+    qa[s] = xs_row_frag(lds_q[slot], c32, s, hh);
+    da[s] = xs_row_frag(lds_do[slot], c32, s, hh);
+    if (s < 4) {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(&lds_nlse[slot][8 * s + 4 * hh]);
+      const f32x4 b = *reinterpret_cast<const f32x4*>(&lds_ndel[slot][8 * s + 4 * hh]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        nl[4 * s + i] = a[i];
+        nd[4 * s + i] = b[i];
+      }
+    }
+  };
 
 #ifdef MVIT_STAMP
   long long stamp_acc[6] = {0, 0, 0, 0, 0, 0};
@@ -1335,7 +1349,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
       pw[j] = pack2(e0, e1);
       dw[j] = pack2(e0 * dp[0][2 * j], e1 * dp[0][2 * j + 1]);
     };
-    int done = 0;
+    BOps pb, db;
 #pragma unroll
     for (int s = 0; s < ND; ++s) {
       if (s == 0) {
@@ -1345,14 +1359,16 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
         mfma32x32_acc(sc[1], qa[s], kf[1][s]);
         mfma32x32_acc(dp[1], da[s], vf[1][s]);
       }
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-        if (done < 8) words(done++);
+      if (s < 4) {
+        words(2 * s);
+        words(2 * s + 1);
+      } else {  // the lane swaps of group 0 under the last two score MFMAs
+        pb = to_b_operands(pw);
+        db = to_b_operands(dw);
+        asm volatile("s_nop 1");
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
-    BOps pb = to_b_operands(pw), db = to_b_operands(dw);
-    asm volatile("s_nop 1");
-    __builtin_amdgcn_sched_barrier(0);
     STAMP(1)
     // ---- phase 3: dV / dK of key group 0 under the vector work of group 1
     unsigned pw1[8], dw1[8];
@@ -1361,21 +1377,23 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
       pw1[j] = pack2(e0, e1);
       dw1[j] = pack2(e0 * dp[1][2 * j], e1 * dp[1][2 * j + 1]);
     };
-    done = 0;
+    BOps pb1, db1;
 #pragma unroll
     for (int d = 0; d < ND; ++d) {
       dv[0][d] = mfma32(dt_[d], pb.lo, dv[0][d]);
       dk[0][d] = mfma32(qt[d], db.lo, dk[0][d]);
       dv[1][d] = mfma32(dt_[d], pb.hi, dv[1][d]);
       dk[1][d] = mfma32(qt[d], db.hi, dk[1][d]);
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-        if (done < 8) words1(done++);
+      if (d < 4) {
+        words1(2 * d);
+        words1(2 * d + 1);
+      } else {
+        pb1 = to_b_operands(pw1);
+        db1 = to_b_operands(dw1);
+        asm volatile("s_nop 1");
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
-    BOps pb1 = to_b_operands(pw1), db1 = to_b_operands(dw1);
-    asm volatile("s_nop 1");
-    __builtin_amdgcn_sched_barrier(0);
     STAMP(2)
     // ---- phase 4: dV / dK of key group 1 under the fragment reads of the next tile; the barrier is waited for while
     // these MFMAs drain
@@ -1385,8 +1403,9 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
       dk[2][d] = mfma32(qt[d], db1.lo, dk[2][d]);
       dv[3][d] = mfma32(dt_[d], pb1.hi, dv[3][d]);
       dk[3][d] = mfma32(qt[d], db1.hi, dk[3][d]);
+      fetch_rows_part(b1, d);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    fetch_rows(b1);
     STAMP(3)
     // tile it+2 (requested in iteration it-1) must have landed before any wave reads it in the next iteration; the
     // loads requested in this iteration (at most five) may stay in flight
@@ -1568,7 +1587,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_wide(const AttnParams p) {
       }
     };
     mask_tail(0);
-    int done = 0;
+    BOps d0;
 #pragma unroll
     for (int s = 0; s < ND; ++s) {
       if (s == 0) {
@@ -1578,38 +1597,42 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_wide(const AttnParams p) {
         mfma32x32_acc(sc[1], ka[s], qf[1][s]);
         mfma32x32_acc(dp[1], va[s], dof[1][s]);
       }
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-        if (done < 8) word(0, done++);
+      if (s < 4) {
+        word(0, 2 * s);
+        word(0, 2 * s + 1);
+      } else {  // the lane swaps of block 0 under the last two score MFMAs
+        d0 = to_b_operands(dw[0]);
+        asm volatile("s_nop 1");
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
-    const BOps d0 = to_b_operands(dw[0]);
-    asm volatile("s_nop 1");
-    __builtin_amdgcn_sched_barrier(0);
     STAMP(1)
     // ---- phase 3: dQ of query block 0 under the vector work of block 1
     mask_tail(1);
-    done = 0;
+    BOps d1;
 #pragma unroll
     for (int d = 0; d < ND; ++d) {
       dq[0][0][d] = mfma32(kt[d], d0.lo, dq[0][0][d]);
       dq[0][1][d] = mfma32(kt[d], d0.hi, dq[0][1][d]);
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-        if (done < 8) word(1, done++);
+      if (d < 4) {
+        word(1, 2 * d);
+        word(1, 2 * d + 1);
+      } else {
+        d1 = to_b_operands(dw[1]);
+        asm volatile("s_nop 1");
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
-    const BOps d1 = to_b_operands(dw[1]);
-    asm volatile("s_nop 1");
-    __builtin_amdgcn_sched_barrier(0);
     STAMP(2)
     // ---- phase 4: dQ of query block 1 under the fragment reads of the next tile
 #pragma unroll
     for (int d = 0; d < ND; ++d) {
       dq[1][0][d] = mfma32(kt[d], d1.lo, dq[1][0][d]);
       dq[1][1][d] = mfma32(kt[d], d1.hi, dq[1][1][d]);
+      ka[d] = xs_row_frag(lds_k[b1], c32, d, hh);
+      va[d] = xs_row_frag(lds_v[b1], c32, d, hh);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    fetch_rows(b1);
     STAMP(3)
     // tile it+2 (requested in iteration it-1) must have landed before any wave reads it in the next iteration
     if (k0 + 3 * BK < L) wait_vmcnt<4>();

@@ -117,15 +117,21 @@ class AttnGeometry:
     order: Optional[torch.Tensor] = None  # device int32 permutation of the segments, longest first (ops.segment_order)
 
 
-def _block_forward(x: torch.Tensor, W: BlockWeights, geo: AttnGeometry, eps: float) -> Tuple[torch.Tensor, tuple]:
+def _block_forward(x: torch.Tensor, W: BlockWeights, geo: AttnGeometry, eps: float,
+                   attn_out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> Tuple[torch.Tensor, tuple]:
+    """``attn_out`` = (o, lse) kept from an earlier run of the same block on the same input: the attention product is
+    then not computed again (the recomputation of a checkpointed block)."""
     S, C = x.shape
     H, hd = geo.nheads, geo.head_dim
     n1, rstd1 = ops.rmsnorm_fwd(x, W.norm1.view(-1), eps)
     qkv = torch.empty(S, 3 * C, dtype=x.dtype, device=x.device)
     ops.gemm(n1, W.wqkv, qkv, epilogue=E.EPI_BIAS, bias=W.bqkv.view(-1))
     ops.rope_(qkv, geo.cos, geo.sin, 2 * H, hd)  # q and k are the first 2*H heads of every row
-    o, lse = ops.attn_fwd(qkv[:, :C], qkv[:, C : 2 * C], qkv[:, 2 * C :], geo.cu, geo.max_seqlen, H, hd, hd**-0.5,
-                          seg_order=geo.order)
+    if attn_out is None:
+        o, lse = ops.attn_fwd(qkv[:, :C], qkv[:, C : 2 * C], qkv[:, 2 * C :], geo.cu, geo.max_seqlen, H, hd, hd**-0.5,
+                              seg_order=geo.order)
+    else:
+        o, lse = attn_out
     x1 = torch.empty_like(x)
     ops.gemm(o, W.wproj, x1, epilogue=E.EPI_BIAS_RES, bias=W.bproj.view(-1), residual=x)
     n2, rstd2 = ops.rmsnorm_fwd(x1, W.norm2.view(-1), eps)
@@ -209,9 +215,15 @@ def _block_backward(dx2: torch.Tensor, x: torch.Tensor, saved: tuple, W: BlockWe
     return dx, grads
 
 
+KEEP_ATTENTION_ABOVE = 64  # segments longer than this (the full-attention layers) keep their attention output when checkpointed
+
+
 class VisionBlockFn(torch.autograd.Function):
     """One transformer block.  With `checkpoint` only the block input is kept and the forward is re-run in
-    the backward (the native counterpart of torch.utils.checkpoint around the block, [tf] modeling_layers.py:79)."""
+    the backward (the native counterpart of torch.utils.checkpoint around the block, [tf] modeling_layers.py:79).
+    A full-attention layer also keeps its attention output and log-sum-exp ([S, C] + [H, S] fp32: 164 MiB at 65,536
+    patches), so the re-run skips the one product whose cost grows with the square of the segment length; the values
+    it would recompute are bit-identical, hence so are the gradients."""
 
     @staticmethod
     def forward(ctx, x, holder, geo: AttnGeometry, eps: float, checkpoint: bool, *params):
@@ -222,6 +234,7 @@ class VisionBlockFn(torch.autograd.Function):
         ctx.gdt = {name: p.dtype for name, p in zip(BLOCK_PARAM_ORDER, params)}
         ctx.x = x
         ctx.saved = None if checkpoint else saved
+        ctx.attn_out = (saved[3], saved[4]) if checkpoint and geo.max_seqlen > KEEP_ATTENTION_ABOVE else None
         return x2
 
     @staticmethod
@@ -232,12 +245,13 @@ class VisionBlockFn(torch.autograd.Function):
         if saved is None:
             ops.recomputing = True
             try:
-                _, saved = _block_forward(x, W, geo, ctx.eps)
+                _, saved = _block_forward(x, W, geo, ctx.eps, ctx.attn_out)
             finally:
                 ops.recomputing = False
         dx, grads = _block_backward(dx2, x, saved, W, geo, ctx.gdt)
         ctx.saved = None
         ctx.x = None
+        ctx.attn_out = None
         return (dx, None, None, None, None) + tuple(grads)
 
 

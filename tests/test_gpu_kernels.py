@@ -384,6 +384,12 @@ def _attn_case(dtype, seglens, H, d, seed=0, qkv_packed=True):
         ([100, 60], 8, 32),
         ([129], 2, 64),
         ([96, 200], 2, 128),
+        # long segments (the 64-rows-per-wave backward kernels): tile multiples, tails of 1 / 31 / 33 rows, short
+        # segments riding in the same launch
+        ([512], 2, 80),
+        ([513, 543], 2, 80),
+        ([576, 1000, 33, 1], 4, 80),
+        ([1200, 77, 640, 607], 3, 80),
     ],
 )
 def test_attention_fwd_bwd(dtype, seglens, H, d):
@@ -431,17 +437,20 @@ def test_attention_segment_order_changes_nothing(dtype):
         ops.attn_fwd(q, k, v, cu, 64, H, d, d**-0.5, seg_order=torch.zeros(2, dtype=torch.int32, device=DEV))
 
 
-def test_attention_sp_share_real_shape():
-    """One rank's share of Ulysses SP=4 attention at its real shape: 65,536 tokens, 4 of the 16 heads, head_dim 80.
+@pytest.mark.parametrize("H", [4, 16])
+def test_attention_sp_share_real_shape(H):
+    """One rank's share of Ulysses SP=4 attention at its real shape: 65,536 tokens, 4 of the 16 heads, head_dim 80
+    (and, with 16 heads, the full-attention layer of the 65,536-patch image as the unsharded tower runs it).
     Windowed layout (64-token windows): everything against the oracle.  Full layer: the oracle's O(L^2) pass is
     out of reach on the host, so sampled query rows (O, lse, dQ) and sampled key rows (dK, dV) are recomputed in
     fp32 from their definitions; the key-row check takes lse and O for the non-sampled rows from the kernel."""
     ops = _ops()
-    L, H, d = 65536, 4, 80
+    L, d = 65536, 80
     scale = d**-0.5
-    _announce("attention bf16 SP share, windows")
-    _attn_case(torch.bfloat16, [64] * 1024, H, d, seed=11)
-    _announce("attention bf16 SP share, full layer")
+    if H == 4:
+        _announce("attention bf16 SP share, windows")
+        _attn_case(torch.bfloat16, [64] * 1024, H, d, seed=11)
+    _announce(f"attention bf16 65,536 tokens x {H} heads, full layer")
     g = torch.Generator().manual_seed(12)
     q, k, v, do = (torch.randn(L, H * d, generator=g).to(torch.bfloat16).to(DEV) for _ in range(4))
     cu = torch.tensor([0, L], dtype=torch.int32, device=DEV)
