@@ -269,3 +269,55 @@ def test_forward_after_a_fused_adam_step_uses_the_updated_weights(dtype, autocas
     sgd.step()
     after_sgd = forward().detach().float().cpu()
     assert max_rel_err(after_sgd, final) > 1e-2
+
+
+def test_windowed_block_on_each_sequence_parallel_share_equals_the_unsharded_block():
+    """One rank's share of a windowed layer under Ulysses sequence parallelism (modeling:492-581): the pack is cut at
+    window boundaries, so a block run on a rank's rows with the rank-local window boundaries and rotary rows needs no
+    exchange.  For sp = 4 every rank's output (and input gradient) must equal the matching rows of the unsharded block
+    bit for bit."""
+    from mi355_vit import ops
+    from mi355_vit import sequence_parallel_utils as spu
+    from mi355_vit.config import Qwen2_5_VLVisionConfig
+    from mi355_vit.modeling import Qwen2_5_VLVisionBlock
+
+    print("[case] windowed block on sp=4 shares", flush=True)
+    torch.manual_seed(7)
+    cfg = Qwen2_5_VLVisionConfig(depth=1, hidden_size=1280, intermediate_size=3420, num_heads=16, out_hidden_size=256, fullatt_block_indexes=[])
+    blk = Qwen2_5_VLVisionBlock(cfg, 0).to(torch.bfloat16).to(DEV)
+    grid = torch.tensor([[1, 18, 22], [2, 8, 12], [1, 34, 16], [1, 4, 4]])
+    _, cu_w = ops.window_index(grid, 2, 112, 14)
+    cu_f = ops.cu_seqlens(grid)
+    lengths = (cu_f[1:] - cu_f[:-1]).tolist()
+    S = sum(lengths)
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(S, 1280, generator=g).to(torch.bfloat16).to(DEV)
+    ang = torch.randn(S, 40, generator=g)
+    emb = torch.cat((ang, ang), dim=-1)
+    cos, sin = emb.cos().to(DEV), emb.sin().to(DEV)
+    gy = torch.randn(S, 1280, generator=g).to(torch.bfloat16).to(DEV)
+
+    xf = x.clone().requires_grad_(True)
+    y_full = blk(xf, cu_seqlens=cu_w.to(DEV), position_embeddings=(cos, sin))
+    y_full.backward(gy)
+    outs, dxs, metas = [], [], []
+    for r in range(4):
+        xr, meta = spu.split_pack_by_sp(x, lengths, r, 4, cu_window_seqlens=cu_w)
+        gr, _ = spu.split_pack_by_sp(gy, lengths, r, 4, cu_window_seqlens=cu_w)
+        cu_local = spu.rebuild_local_cu_seqlens(meta, use_windows=True)
+        cos_r, sin_r, _ = spu.build_local_rope(meta, cos, sin)
+        assert int(cu_local[-1]) == xr.shape[0] == cos_r.shape[0]
+        xr = xr.clone().requires_grad_(True)
+        if xr.shape[0]:
+            yr = blk(xr, cu_seqlens=cu_local.to(DEV), position_embeddings=(cos_r, sin_r))
+            yr.backward(gr)
+            outs.append(yr.detach())
+            dxs.append(xr.grad)
+        else:
+            outs.append(xr.detach())
+            dxs.append(torch.zeros_like(xr))
+        metas.append(meta)
+    lm = [m.local_lengths for m in metas]
+    assert torch.equal(spu.gather_rank_packs(outs, lm), y_full.detach())
+    assert torch.equal(spu.gather_rank_packs(dxs, lm), xf.grad)
+    assert sum(o.shape[0] for o in outs) == S and min(o.shape[0] for o in outs) > 0
