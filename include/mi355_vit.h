@@ -134,8 +134,6 @@ typedef struct mvit_gemm_args {
   int trans_a;   /* 0: A is [M,K] (lda >= K);  1: A is [K,M] (lda >= M) */
   int trans_b;   /* 0: B is [N,K] (ldb >= K);  1: B is [K,N] (ldb >= N) */
   int epilogue;  /* MVIT_EPI_* */
-  int reserved;  /* main-loop variant: 0 = default; 1 = register-staged, 3 = direct-to-LDS with the MFMA shape chosen per
-                    operand layout, 5 / 7 = direct-to-LDS on 16x16x32 / 32x32x16 MFMA only (tuning / tests) */
   int64_t M, N, K;
   const void* A;
   int64_t lda;
@@ -157,7 +155,6 @@ typedef struct mvit_gemm_args {
   int64_t workspace_bytes;
   int split_k;   /* <= 1: one work-group per tile walks all of K.  > 1 (EPI_NONE only): K is cut in split_k slices
                     whose fp32 partial tiles go to `workspace` and are summed by a second kernel (fixed order) */
-  int reserved2; /* tuning: bits 0-7 tile-order panel width (0 = default), bit 9 one work-group per tile; 0 in production */
 } mvit_gemm_args;
 
 /* C[M,N] = epilogue(sum_k A[m,k] * B[n,k]).  Operands must be 16-byte aligned with lda/ldb multiples of

@@ -81,9 +81,6 @@ __device__ __forceinline__ bf16x8 pack8(const f32x4& a, const f32x4& b) {
 __device__ __forceinline__ f32x4 mfma32(const bf16x8& a, const bf16x8& b, const f32x4& c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
-__device__ __forceinline__ f32x4 mfma16(const bf16x4& a, const bf16x4& b, const f32x4& c) {
-  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
-}
 
 template <int ND>
 struct Geo {
@@ -162,26 +159,18 @@ __device__ __forceinline__ void load_rowfrag_lds(RowFrag<ND>& f, const bf16_t* t
 // The 16-wide remainder of head_dim (odd ND) is issued as a 32-wide MFMA whose upper four contraction slots
 // are zero: a v_mfma_f32_16x16x16_bf16 chained onto the accumulator of the 32-wide steps returned wrong sums
 // on gfx950 (also with an all-zero remainder), so that instruction is not used here.
-#ifndef MVIT_TAIL_MODE
-#define MVIT_TAIL_MODE 0
-#endif
 template <int ND>
 __device__ __forceinline__ f32x4 dot_frag(const RowFrag<ND>& a, const RowFrag<ND>& b) {
   using G = Geo<ND>;
   f32x4 c = {0.f, 0.f, 0.f, 0.f};
-#if MVIT_TAIL_MODE == 1
-  if (G::TAIL16) c = mfma16(a.k16, b.k16, c);
-#endif
 #pragma unroll
   for (int ks = 0; ks < G::NK32; ++ks) c = mfma32(a.k32[ks], b.k32[ks], c);
-#if MVIT_TAIL_MODE == 0
   if (G::TAIL16) {
     const bf16_t z = (bf16_t)0.f;
     const bf16x8 ax = {a.k16[0], a.k16[1], a.k16[2], a.k16[3], z, z, z, z};
     const bf16x8 bx = {b.k16[0], b.k16[1], b.k16[2], b.k16[3], z, z, z, z};
     c = mfma32(ax, bx, c);
   }
-#endif
   return c;
 }
 
@@ -510,24 +499,17 @@ __global__ __launch_bounds__(64 * NWAVES, MINW) void attn_fwd_mfma(const AttnPar
 // which lane l holds, for columns l%16 (words 0-3) and 16 + l%16 (words 4-7), the rows
 //     base(G) + {0..3}  and  base(G) + 8 + {0..3},   G = l / 16,  base = {0, 16, 4, 20}[G]
 // in its eight contraction slots; the transposed left factor is read from LDS with the same row mapping.
-// Row statistics ride in the accumulator input of the first MFMA of a chain (a tile of "- stabiliser" values), so
+// Row statistics ride in the accumulator input of the first MFMA of a chain (a tile of "- statistic" values), so
 // exp2 is applied to the MFMA result directly.
-typedef unsigned int u32x8_t __attribute__((ext_vector_type(8)));
-
-__device__ __forceinline__ f32x16 mfma32x32(const bf16x8& a, const bf16x8& b, const f32x16& c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-}
-// acc += a . b on v_mfma_f32_16x16x32_bf16 with the accumulator pinned to the accumulation registers (the compiler
-// otherwise moves accumulators between the two register files).  It does not see an MFMA here: before ordinary
-// instructions touch such an accumulator again, mfma_drain() must have run.
-__device__ __forceinline__ void mfma16_acc(f32x4& acc, const bf16x8& a, const bf16x8& b) {
-  acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
-}
-// d = a . b + c and d += a . b on v_mfma_f32_32x32x16_bf16, all operands in ordinary vector registers (the compiler's own
-// MFMA selection would place results in accumulation registers and copy them back for the vector ALU).  The same rule
-// applies: ordinary instructions may read d only after mfma_drain() or after eleven or more other issue slots.
-// The B operand `b` sits in accumulation registers (see to_acc_regs): an operand that never changes costs no
-// ordinary register that way.
+// A wave that is alone on its SIMD issues about one instruction per seven cycles and hides no latency by itself:
+// matrix and vector instructions are therefore interleaved by hand (__builtin_amdgcn_sched_barrier pins the order),
+// LDS fragments are requested a phase before their use, and tiles reach LDS by direct loads three tiles ahead.
+// d = a . b + c and d += a . b on v_mfma_f32_32x32x16_bf16 with the result in ordinary vector registers (the compiler's
+// own MFMA selection would, in a kernel that uses accumulation registers, place results there and copy them back for
+// the vector ALU).  The compiler does not see an MFMA here and inserts no wait states: ordinary instructions may read
+// d only after mfma_drain() or after eleven or more other issue slots (every use below sits behind at least two
+// further MFMAs).  The B operand `b` sits in accumulation registers (see to_acc_regs): an operand that never changes
+// costs no ordinary register that way.
 __device__ __forceinline__ void mfma32x32_init(f32x16& d, const bf16x8& a, const u32x4& b, const f32x16& c) {
   asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(__builtin_bit_cast(u32x4, a)), "a"(b), "v"(c));
 }
@@ -541,17 +523,6 @@ __device__ __forceinline__ u32x4 to_acc_regs(const bf16x8& v, float* slot) {
   u32x4 r;
   asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=a"(r) : "v"(addr) : "memory");
   return r;
-}
-// acc *= factor for an accumulator that lives in the accumulation registers, without the compiler ever seeing it
-// in an ordinary register (it would then keep a second copy of every accumulator across the whole loop): the four
-// values travel through the lane's own 16-byte LDS slot.  Rare path only; call mfma_drain() first.
-__device__ __forceinline__ void scale_acc(f32x4& acc, float factor, float* slot) {
-  const unsigned addr = (unsigned)(uintptr_t)slot;  // LDS byte address
-  asm volatile("ds_write_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(addr), "a"(acc) : "memory");
-  f32x4 t = *reinterpret_cast<volatile f32x4*>(slot);
-  t *= factor;
-  *reinterpret_cast<volatile f32x4*>(slot) = t;
-  asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=a"(acc) : "v"(addr) : "memory");
 }
 __device__ __forceinline__ void mfma_drain() {
   __builtin_amdgcn_sched_barrier(0);
@@ -572,15 +543,6 @@ __device__ __forceinline__ unsigned pack2(float a, float b) {
 __device__ __forceinline__ void swap16(unsigned& a, unsigned& b) {
   asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
 }
-__device__ __forceinline__ void swap16f(float& a, float& b) {
-  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
-}
-// value held by lane l^32
-__device__ __forceinline__ float other_half(float x) {
-  float a = x, b = x;
-  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
-  return (threadIdx.x & 32) ? a : b;  // the swap put the partner's value into b of the lower half and a of the upper half
-}
 struct BOps {
   bf16x8 lo, hi;  // B operands of the 16x16x32 product for columns l%16 and 16 + l%16 of the 32-column tile
 };
@@ -592,24 +554,6 @@ __device__ __forceinline__ BOps to_b_operands(unsigned (&w)[8]) {
   r.lo = __builtin_bit_cast(bf16x8, a);
   r.hi = __builtin_bit_cast(bf16x8, b);
   return r;
-}
-// A operand (16 x 32, transposed read) of the 16x16x32 product matching to_b_operands: rows base(G)+.. of the
-// 32-row group starting at `row0` of a [row][PITCH] tile, columns 16*d .. 16*d+15.
-template <int PITCH>
-__device__ __forceinline__ bf16x8 tr_block_wide(const bf16_t* tile, int row0, int d, int G, int r) {
-  const int row = row0 + 16 * (G & 1) + 4 * (G >> 1) + (r >> 2);
-  if (PITCH == SWZ) {
-    const int chunk = 2 * d + ((r & 3) >> 1), sub = 4 * (r & 1);
-    return tr_pair(tile + swz_off(row, chunk) + sub, tile + swz_off(row + 8, chunk) + sub);
-  }
-  const bf16_t* a = tile + row * PITCH + 16 * d + 4 * (r & 3);
-  return tr_pair(a, a + 8 * PITCH);
-}
-// Row fragment (A or B operand of the 32x32x16 product) of row `row` of a [row][PITCH] tile: 8 elements at 16*s + 8*h.
-template <int PITCH>
-__device__ __forceinline__ bf16x8 row_frag32(const bf16_t* tile, int row, int s, int h) {
-  if (PITCH == SWZ) return *reinterpret_cast<const bf16x8*>(tile + swz_off(row, 2 * s + h));
-  return *reinterpret_cast<const bf16x8*>(tile + row * PITCH + 16 * s + 8 * h);
 }
 __device__ __forceinline__ bf16x8 scale_frag(bf16x8 v, float c) {
 #pragma unroll
@@ -623,257 +567,6 @@ __device__ __forceinline__ bf16x8 load_frag_global(const bf16_t* p, bool valid) 
   if (valid) v = *reinterpret_cast<const bf16x8*>(p);
   return v;
 }
-__device__ __forceinline__ float max16(const f32x16& s) {
-  float m = max3(s[0], s[1], s[2]);
-  m = max3(m, s[3], s[4]);
-  m = max3(m, s[5], s[6]);
-  m = max3(m, s[7], s[8]);
-  m = max3(m, s[9], s[10]);
-  m = max3(m, s[11], s[12]);
-  m = max3(m, s[13], s[14]);
-  return fmaxf(m, s[15]);
-}
-
-// Forward.  Work-group = 256 queries of one (segment, head).  K / V tiles of 64 keys go through LDS rings of three
-// tiles (tile i+2 is fetched from memory while tile i is used); within the loop a wave handles 32 keys per step and
-// everything a step needs is requested one step earlier: the scores of step t+1 are computed (MFMA) while the softmax
-// of step t runs (VALU), and the LDS fragments of step t+1 are read while step t computes.  The running stabiliser of
-// a row only moves when a score exceeds it by more than TAU (log2 units).
-template <int ND>
-__global__ __launch_bounds__(256, 1) void attn_fwd_wide(const AttnParams p) {
-  static_assert(ND == 5, "the hand-placed instruction order below is laid out for head_dim 80");
-  using G = Geo<ND>;
-  constexpr int HD = G::HD, NT = 256, BNK = 64, PKW = G::PK, PVW = G::PV;
-  constexpr float TAU = 8.f;
-  __shared__ __attribute__((aligned(16))) bf16_t lds_k[3][BNK * PKW];
-  __shared__ __attribute__((aligned(16))) bf16_t lds_v[3][BNK * PVW];
-  __shared__ __attribute__((aligned(16))) float lds_fix[NT * 4];  // one 16-byte slot per lane (scale_acc, to_acc_regs)
-
-  int seg, h;
-  seg_and_head(p, seg, h);
-  const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
-  const int blk_q0 = blockIdx.x * 256;
-  if (blk_q0 >= L) return;
-  const int l = threadIdx.x & 63, wv = threadIdx.x >> 6, hh = l >> 5, c32 = l & 31, G4 = l >> 4, r = l & 15;
-  const int q0 = blk_q0 + wv * 64;
-
-  const bf16_t* Q = static_cast<const bf16_t*>(p.q) + (int64_t)s0 * p.q_stride + (int64_t)h * HD;
-  const bf16_t* K = static_cast<const bf16_t*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD;
-  const bf16_t* V = static_cast<const bf16_t*>(p.v) + (int64_t)s0 * p.v_stride + (int64_t)h * HD;
-
-  const float c = p.scale * LOG2E;
-  // B operands of the score product (column = query 32*qb + l%32, contraction = head-dim 16*s + 8*(l/32) ..), scaled by
-  // softmax_scale * log2(e) and parked in accumulation registers for the whole kernel
-  u32x4 qf[2][ND];
-#pragma unroll
-  for (int qb = 0; qb < 2; ++qb) {
-    const int qi = q0 + 32 * qb + c32;
-#pragma unroll
-    for (int s = 0; s < ND; ++s)
-      qf[qb][s] = to_acc_regs(scale_frag(load_frag_global(Q + (int64_t)qi * p.q_stride + 16 * s + 8 * hh, qi < L), c), lds_fix + threadIdx.x * 4);
-  }
-  f32x4 o[2][2][ND];
-  f32x16 negm[2];
-  float m_run[2], lsum[2];
-#pragma unroll
-  for (int qb = 0; qb < 2; ++qb) {
-    m_run[qb] = 0.f;
-    lsum[qb] = 0.f;
-    negm[qb] = splat16(0.f);
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf)
-#pragma unroll
-      for (int d = 0; d < ND; ++d) o[qb][hf][d] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
-  const bf16x2 ones2 = {(bf16_t)1.f, (bf16_t)1.f};
-
-  TileStager<ND, BNK, PKW, NT> sk;
-  TileStager<ND, BNK, PVW, NT> sv;
-  sk.init(p.k_stride);
-  sv.init(p.v_stride);
-  auto rows_from = [&](int k0) { return max(0, min(BNK, L - k0)); };
-#pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    sk.load(K + (int64_t)t * BNK * p.k_stride, rows_from(t * BNK));
-    sv.load(V + (int64_t)t * BNK * p.v_stride, rows_from(t * BNK));
-    sk.store(lds_k[t]);
-    sv.store(lds_v[t]);
-  }
-  __syncthreads();
-
-  struct Frags {
-    bf16x8 kf[ND], vf[ND];
-  };
-  // LDS fragments of one step: K rows krow0.. of tk (scores of the following step), V rows vrow0.. of tv (this step)
-  auto fetch = [&](Frags& f, const bf16_t* tk, int krow0, const bf16_t* tv, int vrow0) {
-#pragma unroll
-    for (int s = 0; s < ND; ++s) f.kf[s] = row_frag32<PKW>(tk, krow0 + c32, s, hh);
-#pragma unroll
-    for (int d = 0; d < ND; ++d) f.vf[d] = tr_block_wide<PVW>(tv, vrow0, d, G4, r);
-  };
-  // Between two steps: masks the keys past the segment end (only the segment's last step can have any), then
-  // moves the stabiliser of rows whose scores outgrew it (rare: taken when any lane of the wave asks for it).
-  auto settle = [&](f32x16 (&sc)[2], float mx0, float mx1, int key0, bool first) {
-    if (key0 + 32 > L) {
-      asm volatile("" ::: "memory");  // keeps this rare block a branch (as selects it would run on every step)
-#pragma unroll
-      for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i)
-          if (key0 + 8 * (i >> 2) + 4 * hh + (i & 3) >= L) sc[qb][i] = -INFINITY;
-      mx0 = max16(sc[0]);
-      mx1 = max16(sc[1]);
-    }
-    if (__builtin_amdgcn_ballot_w64(first || mx0 > TAU || mx1 > TAU) == 0) return;
-    mfma_drain();  // the output accumulators are about to be read by ordinary instructions
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-      const float mine = qb == 0 ? mx0 : mx1;
-      const float mfull = fmaxf(mine, other_half(mine));  // over all 32 keys of the step
-      const bool grow = first || mfull > TAU;
-      const float delta = grow ? mfull : 0.f;
-      const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);
-      m_run[qb] += delta;
-      negm[qb] = splat16(-m_run[qb]);
-      lsum[qb] *= alpha;
-      float a0 = alpha, a1 = alpha;
-      swap16f(a0, a1);  // a0: factor of query 32*qb + l%16, a1: of query 32*qb + 16 + l%16
-#pragma unroll
-      for (int d = 0; d < ND; ++d) {
-        scale_acc(o[qb][0][d], a0, lds_fix + threadIdx.x * 4);
-        scale_acc(o[qb][1][d], a1, lds_fix + threadIdx.x * 4);
-      }
-#pragma unroll
-      for (int i = 0; i < 16; ++i) sc[qb][i] -= delta;
-    }
-    mfma_drain();
-  };
-  // One 32-key step: softmax numerators of `cur` (scores, ready) -> row sums and O^T += V^T P^T with the V fragments
-  // of `f`, while the scores of the following step are computed from the K fragments of `f` into `nxt` and the
-  // fragments of the following step are read into `fn` (get_next).  The instruction stream alternates matrix and
-  // vector work by hand (a wave is alone on its SIMD): score MFMAs run under the first query block's exp / pack, the
-  // first block's PV MFMAs under the second block's, the second block's PV MFMAs under the row maxima of the new
-  // scores (returned in mx0, mx1).
-  auto step = [&](f32x16 (&cur)[2], f32x16 (&nxt)[2], const Frags& f, auto get_next, float& mx0, float& mx1) {
-    get_next();
-    unsigned w[2][8];
-    auto word = [&](int qb, int j) {
-      w[qb][j] = pack2(__builtin_amdgcn_exp2f(cur[qb][2 * j]), __builtin_amdgcn_exp2f(cur[qb][2 * j + 1]));
-      lsum[qb] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w[qb][j]), ones2, lsum[qb], false);
-    };
-    int done0 = 0, done1 = 0;
-#pragma unroll
-    for (int s = 0; s < ND; ++s) {
-      if (s == 0) {
-        mfma32x32_init(nxt[0], f.kf[0], qf[0][0], negm[0]);
-        mfma32x32_init(nxt[1], f.kf[0], qf[1][0], negm[1]);
-      } else {
-        mfma32x32_acc(nxt[0], f.kf[s], qf[0][s]);
-        mfma32x32_acc(nxt[1], f.kf[s], qf[1][s]);
-      }
-      if (s < 3) {
-#pragma unroll
-        for (int j = 0; j < 3; ++j)
-          if (done0 < 8) word(0, done0++);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          if (done1 < 8) word(1, done1++);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    const BOps p0 = to_b_operands(w[0]);
-    asm volatile("s_nop 1");
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int d = 0; d < ND; ++d) {
-      mfma16_acc(o[0][0][d], f.vf[d], p0.lo);
-      mfma16_acc(o[0][1][d], f.vf[d], p0.hi);
-      if (done1 < 8) word(1, done1++);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    const BOps p1 = to_b_operands(w[1]);
-    asm volatile("s_nop 1");
-    __builtin_amdgcn_sched_barrier(0);
-    float ma = nxt[0][0], mb = nxt[1][0];
-#pragma unroll
-    for (int d = 0; d < ND; ++d) {
-      mfma16_acc(o[1][0][d], f.vf[d], p1.lo);
-      mfma16_acc(o[1][1][d], f.vf[d], p1.hi);
-#pragma unroll
-      for (int i = 1 + 3 * d; i < 1 + 3 * (d + 1); ++i) {
-        ma = fmaxf(ma, nxt[0][i]);
-        mb = fmaxf(mb, nxt[1][i]);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    mx0 = ma;
-    mx1 = mb;
-  };
-
-  f32x16 sa[2], sb[2];
-  Frags fa, fb;
-  float mx0, mx1;
-  {  // scores of the first 32 keys, nothing to overlap them with
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-      for (int s = 0; s < ND; ++s) {
-        const bf16x8 kf = row_frag32<PKW>(lds_k[0], c32, s, hh);
-        if (s == 0) mfma32x32_init(sa[qb], kf, qf[qb][0], negm[qb]);
-        else mfma32x32_acc(sa[qb], kf, qf[qb][s]);
-      }
-    mfma_drain();
-    settle(sa, max16(sa[0]), max16(sa[1]), 0, true);
-  }
-  fetch(fa, lds_k[0], 32, lds_v[0], 0);
-  int b0 = 0, b1 = 1, b2 = 2;  // ring slots of this tile, the next one, and the one being filled
-  for (int k0 = 0; k0 < L; k0 += BNK) {
-    sk.load(K + (int64_t)(k0 + 2 * BNK) * p.k_stride, rows_from(k0 + 2 * BNK));
-    sv.load(V + (int64_t)(k0 + 2 * BNK) * p.v_stride, rows_from(k0 + 2 * BNK));
-    // step A: keys k0 .. k0+31 (scores in sa); the scores of keys k0+32 .. k0+63 are computed alongside
-    step(sa, sb, fa, [&] { fetch(fb, lds_k[b1], 0, lds_v[b0], 32); }, mx0, mx1);
-    if (k0 + 32 < L) {
-      settle(sb, mx0, mx1, k0 + 32, false);
-      // step B: keys k0+32 .. k0+63 (scores in sb); the scores of the next tile's first 32 keys alongside
-      step(sb, sa, fb, [&] { fetch(fa, lds_k[b1], 32, lds_v[b1], 0); }, mx0, mx1);
-    }
-    sk.store(lds_k[b2]);  // slot b2 held tile i-1: last read before the barrier that ended the previous iteration
-    sv.store(lds_v[b2]);
-    if (k0 + BNK < L) settle(sa, mx0, mx1, k0 + BNK, false);
-    __syncthreads();
-    const int t = b0;
-    b0 = b1;
-    b1 = b2;
-    b2 = t;
-  }
-  mfma_drain();
-
-  bf16_t* O = static_cast<bf16_t*>(p.out) + (int64_t)s0 * p.o_stride + (int64_t)h * HD;
-#pragma unroll
-  for (int qb = 0; qb < 2; ++qb) {
-    const float lt = lsum[qb] + other_half(lsum[qb]);
-    float i0 = 1.f / lt, i1 = i0;
-    swap16f(i0, i1);
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-      const int qi = q0 + 32 * qb + 16 * hf + r;
-      if (qi < L) {
-        const float inv = hf == 0 ? i0 : i1;
-#pragma unroll
-        for (int d = 0; d < ND; ++d) {
-          bf16x4 ov;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) ov[i] = (bf16_t)(o[qb][hf][d][i] * inv);
-          *reinterpret_cast<bf16x4*>(O + (int64_t)qi * p.o_stride + 16 * d + 4 * G4) = ov;
-        }
-      }
-    }
-    const int qi = q0 + 32 * qb + c32;
-    if (hh == 0 && qi < L) p.lse[(int64_t)h * p.total + s0 + qi] = (m_run[qb] + __builtin_amdgcn_logf(lt)) * LN2;
-  }
-}
-
 // delta[h, s] = sum_d O[s,h,d] * dO[s,h,d].  One lane per (row, head), 16-byte loads; neighbouring lanes take
 // neighbouring heads of the same row, so a wave sweeps contiguous memory.
 template <typename T>
@@ -1312,19 +1005,11 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
     }
   };
 
-#ifdef MVIT_STAMP
-  long long stamp_acc[6] = {0, 0, 0, 0, 0, 0};
-  long long t_prev = __builtin_readcyclecounter();
-#define STAMP(i) { __builtin_amdgcn_sched_barrier(0); long long t_now = __builtin_readcyclecounter(); stamp_acc[i] += t_now - t_prev; t_prev = t_now; __builtin_amdgcn_sched_barrier(0); }
-#else
-#define STAMP(i)
-#endif
   int it = 0;
   for (int qs = 0; qs < L; qs += BQ, ++it) {
     const int b0 = it & 3, b1 = (it + 1) & 3, b3 = (it + 3) & 3;
     // tile it+3 is requested into the slot that tile it-1 left (every wave is past the barrier that ended iteration it-1)
     request_tile(qs + 3 * BQ, b3);
-    STAMP(5)
     // ---- phase 1: score products of key group 0; the transposed left factors that phase 3 needs are read from LDS
     // between the MFMAs
     bf16x8 qt[ND], dt_[ND];
@@ -1341,7 +1026,6 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
       dt_[s] = xs_tr_block(lds_do[b0], s, G4, r);
       __builtin_amdgcn_sched_barrier(0);
     }
-    STAMP(0)
     // ---- phase 2: score products of key group 1 under the vector work of group 0
     unsigned pw[8], dw[8];
     auto words = [&](int j) {
@@ -1369,7 +1053,6 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    STAMP(1)
     // ---- phase 3: dV / dK of key group 0 under the vector work of group 1
     unsigned pw1[8], dw1[8];
     auto words1 = [&](int j) {
@@ -1394,7 +1077,6 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    STAMP(2)
     // ---- phase 4: dV / dK of key group 1 under the fragment reads of the next tile; the barrier is waited for while
     // these MFMAs drain
 #pragma unroll
@@ -1406,22 +1088,14 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
       fetch_rows_part(b1, d);
       __builtin_amdgcn_sched_barrier(0);
     }
-    STAMP(3)
     // tile it+2 (requested in iteration it-1) must have landed before any wave reads it in the next iteration; the
     // loads requested in this iteration (at most five) may stay in flight
     if (qs + 3 * BQ < L) wait_vmcnt<5>();
     else wait_vmcnt<0>();
     fix_tail(qs + 2 * BQ, (it + 2) & 3);
     __syncthreads();
-    STAMP(4)
   }
 
-#ifdef MVIT_STAMP
-  if (blockIdx.x == 3 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 64) {
-    printf("stamps (ticks, %d iterations): ph1 %lld ph2 %lld ph3 %lld ph4 %lld barrier %lld store %lld\n", (L + BQ - 1) / BQ,
-           stamp_acc[0], stamp_acc[1], stamp_acc[2], stamp_acc[3], stamp_acc[4], stamp_acc[5]);
-  }
-#endif
   bf16_t* DK = static_cast<bf16_t*>(p.dk) + (int64_t)s0 * p.dk_stride + (int64_t)h * HD;
   bf16_t* DV = static_cast<bf16_t*>(p.dv) + (int64_t)s0 * p.dv_stride + (int64_t)h * HD;
 #pragma unroll
@@ -1545,15 +1219,10 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_wide(const AttnParams p) {
   fetch_rows(0);
 
   f32x16 sc[2], dp[2];  // per query block: S^T - lse2 and dP^T - delta, lane = query l%32, register i = key 8*(i/4) + 4*(l/32) + i%4
-#ifdef MVIT_STAMP
-  long long stamp_acc[6] = {0, 0, 0, 0, 0, 0};
-  long long t_prev = __builtin_readcyclecounter();
-#endif
   int it = 0;
   for (int k0 = 0; k0 < L; k0 += BK, ++it) {
     const int b0 = it & 3, b1 = (it + 1) & 3, b3 = (it + 3) & 3;
     request_tile(k0 + 3 * BK, b3);
-    STAMP(5)
     const int valid = L - k0;  // keys of this tile inside the segment (>= 1)
     // ---- phase 1: score products of query block 0; K^T fragments for the dQ products are read between the MFMAs
     bf16x8 kt[ND];
@@ -1569,7 +1238,6 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_wide(const AttnParams p) {
       kt[s] = xs_tr_block(lds_k[b0], s, G4, r);
       __builtin_amdgcn_sched_barrier(0);
     }
-    STAMP(0)
     // ---- phase 2: score products of query block 1 under the vector work of block 0
     unsigned dw[2][8];
     auto word = [&](int qb, int j) {
@@ -1606,7 +1274,6 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_wide(const AttnParams p) {
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    STAMP(1)
     // ---- phase 3: dQ of query block 0 under the vector work of block 1
     mask_tail(1);
     BOps d1;
@@ -1623,7 +1290,6 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_wide(const AttnParams p) {
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    STAMP(2)
     // ---- phase 4: dQ of query block 1 under the fragment reads of the next tile
 #pragma unroll
     for (int d = 0; d < ND; ++d) {
@@ -1633,19 +1299,11 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_wide(const AttnParams p) {
       va[d] = xs_row_frag(lds_v[b1], c32, d, hh);
       __builtin_amdgcn_sched_barrier(0);
     }
-    STAMP(3)
     // tile it+2 (requested in iteration it-1) must have landed before any wave reads it in the next iteration
     if (k0 + 3 * BK < L) wait_vmcnt<4>();
     else wait_vmcnt<0>();
     __syncthreads();
-    STAMP(4)
   }
-#ifdef MVIT_STAMP
-  if (blockIdx.x == 3 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 64) {
-    printf("dq stamps (ticks, %d iterations): ph1 %lld ph2 %lld ph3 %lld ph4 %lld barrier %lld request %lld\n", (L + BK - 1) / BK,
-           stamp_acc[0], stamp_acc[1], stamp_acc[2], stamp_acc[3], stamp_acc[4], stamp_acc[5]);
-  }
-#endif
 
   bf16_t* DQ = static_cast<bf16_t*>(p.dq) + (int64_t)s0 * p.dq_stride + (int64_t)h * HD;
 #pragma unroll
@@ -2198,12 +1856,6 @@ int launch_fwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
     if constexpr (ND <= 5) hipLaunchKernelGGL((attn_fwd_mfma<ND, 2, 64, false, 2, 4>), grid, 128, 0, s, pw);
   } else if (nw == 1) hipLaunchKernelGGL((attn_fwd_mfma<ND, 1, 64, false>), grid, 64, 0, s, p);
   else if (nw == 2) hipLaunchKernelGGL((attn_fwd_mfma<ND, 2, 64, false>), grid, 128, 0, s, p);
-  else if (ND == 5 && max_seqlen >= WIDE_MIN_SEQLEN && false) {
-    AttnParams pl = p;
-    pl.seg_major = 1;
-    dim3 gl((unsigned)((max_seqlen + 255) / 256), (unsigned)p.nheads, (unsigned)n_seg);
-    if constexpr (ND == 5) hipLaunchKernelGGL((attn_fwd_wide<ND>), gl, 256, 0, s, pl);
-  }
   else if constexpr (ND <= 5) {
     // long segments: 8 waves x 32 queries, <= 128 registers, so that four waves share a SIMD and cover each
     // other's MFMA -> softmax -> MFMA dependency stalls

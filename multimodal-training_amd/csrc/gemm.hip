@@ -1,10 +1,11 @@
 // MFMA GEMM for gfx950 with fused epilogues:  C[M,N] = epi( sum_k A[m,k] * B[n,k] ).
 //
-// Main loops (selected by the host; mvit_gemm_args.reserved, 0 = default):
-//   3: bf16 default.  256x256 tile, 8 waves of 128x64 (4x2 MFMA 32x32x16 tiles each), BK = 32, four LDS stages
-//      filled by direct global -> LDS loads (see gemm_dl_kernel).
-//   1: 256x256 tile, 8 waves, BK = 64 (fp32: 16), global -> registers -> LDS, double-buffered LDS, one barrier
-//      per K step.  The fp32 parity path (v_mfma_f32_32x32x2_f32) and the fallback for huge leading dimensions.
+// Main loops:
+//   bf16: 256x256 tile, 8 waves of 128x64 (4x2 MFMA 32x32x16 tiles each), BK = 32, four LDS stages filled by direct
+//      global -> LDS loads (see gemm_dl_kernel).
+//   fp32 (the parity path, v_mfma_f32_32x32x2_f32), and bf16 operands whose row pitch exceeds 2^22 elements (the
+//      direct loads use 32-bit lane offsets): 256x256 tile, 8 waves, BK = 64 (fp32: 16), global -> registers -> LDS,
+//      double-buffered LDS, one barrier per K step (gemm_kernel).
 // Operands whose contraction index is contiguous in memory are staged as [row][k] and read with 16-byte LDS
 // loads; operands whose contraction index is the slow dimension (dgrad's weight, both operands of wgrad) are
 // staged as [k][row] exactly as they lie in memory and read with ds_read_b64_tr_b16, which hands each lane 4
@@ -39,7 +40,6 @@ struct GemmParams {
   float* workspace;   // [split_k][M][N] fp32 partial sums when split_k > 1
   int vec_ok;         // every epilogue pointer / stride allows 16-byte accesses
   float* colsum;      // SWIGLU_BWD: per-tile-row column sums of the output, [tiles_m][ldc] (null: not wanted)
-  int flags;          // tuning switches: 2 = one work-group per tile instead of persistent work-groups
   int panel_w;        // tiles are walked in panels of this many tile columns (M fastest across a panel's rows)
 };
 
@@ -1108,7 +1108,7 @@ int launch_dl(const GemmParams& p, hipStream_t stream) {
     n_cu = v / 8 * 8 > 0 ? v / 8 * 8 : 8;
   }
   const int want = ((total + 7) / 8) * 8;
-  const int grid = (want < n_cu || (p.flags & 2)) ? want : n_cu;
+  const int grid = want < n_cu ? want : n_cu;
   hipLaunchKernelGGL(kern, grid, D::NTHREADS, lds, stream, p);
   MVIT_CHECK_LAUNCH("gemm");
   if (p.split_k > 1) {
@@ -1123,17 +1123,13 @@ int launch_dl(const GemmParams& p, hipStream_t stream) {
 template <typename T, typename TO, bool TA, bool TB, int EPI>
 int launch_var(int var, const GemmParams& p, hipStream_t s) {
   if constexpr (sizeof(T) == 2) {
-    // default: v_mfma_f32_16x16x32_bf16 for the plain GEMMs with an operand behind the transposing LDS read
-    // (weight gradients +6 %, input gradients +1 % on real data), v_mfma_f32_32x32x16_bf16 for the forward GEMMs
-    // (both operands row-major: 3-5 % faster that way) and for the fused backward epilogues; 5 / 7 force one shape
+    // direct-to-LDS main loop: v_mfma_f32_16x16x32_bf16 for the plain GEMMs with an operand behind the transposing
+    // LDS read (weight gradients +6 %, input gradients +1 % on real data), v_mfma_f32_32x32x16_bf16 for the forward
+    // GEMMs (both operands row-major: 3-5 % faster that way) and for the fused backward epilogues
     constexpr int NS = 4;
     if (var == 3) return (TB && EPI == MVIT_EPI_NONE) ? launch_dl<TO, TA, TB, EPI, NS, 8, true>(p, s) : launch_dl<TO, TA, TB, EPI, NS, 8>(p, s);
-    if (var == 5) return launch_dl<TO, TA, TB, EPI, NS, 8, true>(p, s);
-    if (var == 7) return launch_dl<TO, TA, TB, EPI, NS, 8>(p, s);
-
   }
-  if (var == 1 || var >= 3) return launch<T, TO, TA, TB, EPI, 1>(p, s);
-  return launch<T, TO, TA, TB, EPI, 1>(p, s);
+  return launch<T, TO, TA, TB, EPI, 1>(p, s);  // register-staged main loop: fp32, and bf16 operands whose row pitch exceeds 32-bit lane offsets
 }
 
 template <typename T, typename TO, bool TA, bool TB>
@@ -1207,16 +1203,13 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
   const size_t es = a->dtype == MVIT_BF16 ? 2 : 4, eo = a->out_dtype == MVIT_BF16 ? 2 : 4;
   p.vec_ok = vec16(a->C, a->ldc, eo) && vec16(a->R, a->ldr, es) && vec16(a->aux, a->ldaux, es) && vec16(a->bias, 0, es) &&
              vec16(a->bias2, 0, es) && (a->aux_off * (int64_t)(es < eo ? es : eo)) % 16 == 0;
-  int var = (a->reserved == 1 || a->reserved == 3 || a->reserved == 5 || a->reserved == 7) ? a->reserved : 3;  // 0 (or anything else) = default
-  if (var >= 3 && (a->lda > (1ll << 22) || a->ldb > (1ll << 22))) var = 1;  // 32-bit lane offsets  // tile / wave layout, see Waves<>
+  const int var = (a->lda > (1ll << 22) || a->ldb > (1ll << 22)) ? 1 : 3;  // 3: direct-to-LDS loads (32-bit lane offsets); 1: register-staged
   const int BM = 256, BN = 256;
   const int n_per_block = (epi == MVIT_EPI_SWIGLU) ? BN / 2 : BN;
   const int64_t tm = (a->M + BM - 1) / BM, tn = (a->N + n_per_block - 1) / n_per_block;
   MVIT_REQUIRE(tm * tn < (1ll << 30), "gemm: too many tiles");
   p.tiles_m = (int)tm; p.tiles_n = (int)tn;
   p.panel_w = tn <= 6 ? (int)tn : 4;
-  p.flags = (a->reserved2 >> 8) & 0xff;
-  if ((a->reserved2 & 0xff) > 0) p.panel_w = (a->reserved2 & 0xff) < tn ? (a->reserved2 & 0xff) : (int)tn;  // tuning override
   p.split_k = 1; p.k_chunk = a->K; p.workspace = nullptr;
   p.colsum = nullptr;
   if (epi == MVIT_EPI_SWIGLU_BWD && a->workspace) {

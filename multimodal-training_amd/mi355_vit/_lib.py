@@ -19,7 +19,7 @@ _vp, _i64, _i32, _f32 = C.c_void_p, C.c_int64, C.c_int, C.c_float
 
 class GemmArgs(C.Structure):
     _fields_ = [
-        ("dtype", _i32), ("out_dtype", _i32), ("trans_a", _i32), ("trans_b", _i32), ("epilogue", _i32), ("reserved", _i32),
+        ("dtype", _i32), ("out_dtype", _i32), ("trans_a", _i32), ("trans_b", _i32), ("epilogue", _i32),
         ("M", _i64), ("N", _i64), ("K", _i64),
         ("A", _vp), ("lda", _i64),
         ("B", _vp), ("B2", _vp), ("ldb", _i64),
@@ -27,7 +27,7 @@ class GemmArgs(C.Structure):
         ("C", _vp), ("ldc", _i64),
         ("R", _vp), ("ldr", _i64),
         ("aux", _vp), ("ldaux", _i64), ("aux_off", _i64),
-        ("workspace", _vp), ("workspace_bytes", _i64), ("split_k", _i32), ("reserved2", _i32),
+        ("workspace", _vp), ("workspace_bytes", _i64), ("split_k", _i32),
     ]
 
 

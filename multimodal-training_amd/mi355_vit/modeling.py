@@ -150,9 +150,11 @@ class Qwen2_5_VLVisionBlock(nn.Module):
             if position_embeddings is None:
                 emb = torch.cat((rotary_pos_emb, rotary_pos_emb), dim=-1)
                 position_embeddings = (emb.cos(), emb.sin())
-            lengths = cu_seqlens[1:] - cu_seqlens[:-1]
-            max_seqlen = int(lengths.max().item()) if lengths.numel() else 0  # host sync, as in the reference (:433)
+            cu_host = cu_seqlens.detach().cpu()  # host sync, as in the reference (:433)
+            lengths = cu_host[1:] - cu_host[:-1]
+            max_seqlen = int(lengths.max()) if lengths.numel() else 0
             order = ops.segment_order(lengths)
+            ops.check_segments(cu_host, hidden_states.shape[0], max_seqlen, order)
             geo = AttnGeometry(
                 cu_seqlens.to(device=hidden_states.device, dtype=torch.int32).contiguous(), max_seqlen,
                 self.attn.num_heads, self.attn.head_dim,
@@ -187,6 +189,8 @@ class _TowerPlan:
         self.max_window = int((cu_w[1:] - cu_w[:-1]).max()) if cu_w.numel() > 1 else 0
         self.max_full = int((cu_f[1:] - cu_f[:-1]).max()) if cu_f.numel() > 1 else 0
         order_w, order_f = ops.segment_order(cu_w[1:] - cu_w[:-1]), ops.segment_order(cu_f[1:] - cu_f[:-1])
+        ops.check_segments(cu_w, S, self.max_window, order_w)
+        ops.check_segments(cu_f, S, self.max_full, order_f)
         self.order_window = None if order_w is None else order_w.to(device)
         self.order_full = None if order_f is None else order_f.to(device)
 

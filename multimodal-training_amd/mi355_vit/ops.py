@@ -16,9 +16,6 @@ from ._lib import BF16, F32, GemmArgs
 _DT = {torch.float32: F32, torch.bfloat16: BF16}
 N_PARTIAL = 1024  # work-groups (= partial rows) of the RMSNorm backward: 4 per CU keep enough loads in flight
 
-GEMM_PANEL = int(_os.environ.get("MI355_VIT_GEMM_PANEL", "0"))  # bits 0-7: tile-order panel width override (0: library default); bits 8-15: tuning switches
-GEMM_VARIANT = int(_os.environ.get("MI355_VIT_GEMM_VARIANT", "0"))  # GEMM main loop: 0 default, 1 register-staged, 3 direct-to-LDS, 5 / 7 one MFMA shape only
-
 _trace = None  # optional list collecting (tag, info, start_event, end_event) per tagged launch
 recomputing = False  # True while a checkpointed block re-runs its forward inside the backward (marks traced launches)
 
@@ -308,9 +305,8 @@ def gemm(
         raise ValueError(f"gemm: out {tuple(out.shape)} too small for M={M}, N={N}")
     args = GemmArgs()
     args.dtype, args.out_dtype = dt(a), dt(out)
-    args.trans_a, args.trans_b, args.epilogue, args.reserved = int(trans_a), int(trans_b), epilogue, GEMM_VARIANT
+    args.trans_a, args.trans_b, args.epilogue = int(trans_a), int(trans_b), epilogue
     args.M, args.N, args.K = M, N, K
-    args.reserved2 = GEMM_PANEL
     args.A, args.lda = a.data_ptr(), a.stride(0)
     args.B, args.ldb = b.data_ptr(), b.stride(0)
     if b2 is not None:
@@ -403,6 +399,26 @@ def segment_order(lengths: torch.Tensor) -> Optional[torch.Tensor]:
     return torch.sort(ln, descending=True, stable=True).indices.to(torch.int32).contiguous()
 
 
+def check_segments(cu_host: torch.Tensor, total: int, max_seqlen: int, seg_order_host: Optional[torch.Tensor] = None) -> None:
+    """Host-side validation of an attention segment list (the kernels trust it): ``cu_host`` (a CPU tensor) must start
+    at 0, never decrease and end at ``total``; no segment may be longer than ``max_seqlen`` (rows beyond it would be
+    left unwritten); ``seg_order_host`` must be a permutation of the segments.  Raises ValueError."""
+    cu = cu_host.detach().to("cpu", torch.int64)
+    if cu.dim() != 1 or cu.numel() < 1 or int(cu[0]) != 0:
+        raise ValueError("attn: cu_seqlens must be a 1-D list starting at 0")
+    lens = cu[1:] - cu[:-1]
+    if lens.numel() and int(lens.min()) < 0:
+        raise ValueError("attn: cu_seqlens must not decrease")
+    if int(cu[-1]) != total:
+        raise ValueError(f"attn: cu_seqlens ends at {int(cu[-1])} but the inputs hold {total} rows")
+    if lens.numel() and int(lens.max()) > max_seqlen:
+        raise ValueError(f"attn: max_seqlen {max_seqlen} is smaller than the longest segment ({int(lens.max())})")
+    if seg_order_host is not None:
+        o = seg_order_host.detach().to("cpu", torch.int64)
+        if o.numel() != lens.numel() or not torch.equal(torch.sort(o).values, torch.arange(lens.numel())):
+            raise ValueError("attn: seg_order must be a permutation of the segments")
+
+
 def _order_ptr(seg_order: Optional[torch.Tensor], cu_seqlens: torch.Tensor) -> Optional[int]:
     if seg_order is None:
         return None
@@ -414,7 +430,9 @@ def _order_ptr(seg_order: Optional[torch.Tensor], cu_seqlens: torch.Tensor) -> O
 def attn_fwd(q, k, v, cu_seqlens: torch.Tensor, max_seqlen: int, nheads: int, head_dim: int, scale: float, out: Optional[torch.Tensor] = None,
              seg_order: Optional[torch.Tensor] = None):
     """q, k, v: [S, nheads*head_dim] views (row strides free).  Returns (o [S, nheads*head_dim], lse [nheads, S]).
-    ``seg_order``: optional scheduling order of the segments (see segment_order); results do not depend on it."""
+    ``seg_order``: optional scheduling order of the segments (see segment_order); results do not depend on it.
+    ``cu_seqlens``, ``max_seqlen`` and ``seg_order`` live on the device and are trusted as they are (checking them
+    here would cost a read-back per call): callers validate their host copies once with ``check_segments``."""
     S = q.shape[0]
     if cu_seqlens.dtype != torch.int32 or cu_seqlens.device != q.device or not cu_seqlens.is_contiguous():
         raise ValueError("attn: cu_seqlens must be a contiguous int32 tensor on the inputs' device")

@@ -163,3 +163,18 @@ def test_trainer_config_resolution():
     b = next(synthetic_batches([[1, 4, 4], [2, 2, 6]], 0, 1176))
     assert b["pixel_values"].shape == (40, 1176) and b["image_grid_thw"].tolist() == [[1, 4, 4], [2, 2, 6]] and b["sample_index"] == 0
     assert tr._get_torch_dtype("float32") == torch.float32 and tr._get_torch_dtype("nonsense") == torch.bfloat16
+
+
+def test_segment_lists_are_validated_on_the_host():
+    import torch
+
+    from mi355_vit import ops
+
+    ops.check_segments(torch.tensor([0, 4, 4, 9]), 9, 5, torch.tensor([2, 0, 1]))
+    for cu, total, mx, order in (([1, 4], 4, 4, None), ([0, 5, 3], 3, 5, None), ([0, 4], 5, 4, None), ([0, 4, 9], 9, 4, None),
+                                 ([0, 4, 9], 9, 5, [0, 0]), ([0, 4, 9], 9, 5, [0])):
+        try:
+            ops.check_segments(torch.tensor(cu), total, mx, None if order is None else torch.tensor(order))
+        except ValueError:
+            continue
+        raise AssertionError(f"accepted {cu}, total {total}, max {mx}, order {order}")

@@ -498,3 +498,22 @@ def test_attention_softmax_invariants():
     v3[300:] = 1
     o2, _ = ops.attn_fwd(q, k2, v3, cu, 400, H, d, d**-0.5)
     assert torch.equal(o1[:300], o2[:300])
+
+
+def test_gemm_bf16_with_a_row_pitch_beyond_32_bit_lane_offsets():
+    """Operands whose rows lie more than 2^22 elements apart take the register-staged bf16 main loop (the direct
+    global -> LDS loads address a tile with 32-bit lane offsets): same results as the dense layout."""
+    ops = _ops()
+    _announce("gemm bf16, huge row pitch")
+    M, N, K, pitch = 40, 300, 264, (1 << 22) + 8
+    a = _rand((M, K), torch.bfloat16, 21)
+    b = _rand((N, K), torch.bfloat16, 22)
+    big = torch.zeros(M * pitch, dtype=torch.bfloat16, device=DEV)
+    av = big.as_strided((M, K), (pitch, 1))
+    av.copy_(a.to(DEV))
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.gemm(av, b.to(DEV), out)
+    dense = torch.empty_like(out)
+    ops.gemm(a.to(DEV), b.to(DEV), dense)
+    ref = a.float() @ b.float().t()
+    assert max_rel_err(out, ref) < TOL[torch.bfloat16] and max_rel_err(dense, ref) < TOL[torch.bfloat16]
