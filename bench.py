@@ -102,7 +102,9 @@ def summarise_trace(records, cfg_kw, dtype):
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, scaled by what the same
 # counters read for a 1 GiB device copy: x2.000 and x1.000), keyed by (workload, trace tag).  The weight-gradient
 # launch is the GEMM kernel (544.2 MB) plus its split-K reduction (98.4 MB).
-MEASURED_TRAFFIC_BYTES = {("cfg2", "gemm_tt_epi0"): 642.6e6}
+# The full-attention backward launch of cfg3 is the dK/dV kernel (4.91 GB read + 0.34 GB written) plus the dQ kernel
+# (4.84 GB + 0.17 GB) plus the two small preparation kernels (0.5 GB): profiles/attn_cfg3_pmc.txt.
+MEASURED_TRAFFIC_BYTES = {("cfg2", "gemm_tt_epi0"): 642.6e6, ("cfg3", "attn_bwd_full"): 10.8e9}
 
 KERNEL_NAMES = {
     "gemm_nn_epi0": "gemm_dl_kernel<TO, TA=false, TB=false, EPI=NONE>",
