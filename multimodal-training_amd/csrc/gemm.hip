@@ -110,15 +110,41 @@ __device__ __forceinline__ void unpack8(const T __attribute__((ext_vector_type(8
 #pragma unroll
   for (int e = 0; e < 8; ++e) v[e] = (float)x[e];
 }
+// Epilogue outputs and per-element epilogue inputs are touched once per launch: they are stored / loaded with the
+// non-temporal hint, so that they do not push the operand panels of the tiles in flight out of the XCD's L2 (a round of
+// 32 output tiles is as large as that L2; with plain stores the main loop after an epilogue ran 18 % slower).
+typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void store8(bf16_t* p, const float* v) {
   bf16x8 x;
 #pragma unroll
   for (int e = 0; e < 8; ++e) x[e] = (bf16_t)v[e];
-  *reinterpret_cast<bf16x8*>(p) = x;
+  __builtin_nontemporal_store(__builtin_bit_cast(u32x4_t, x), reinterpret_cast<u32x4_t*>(p));
 }
 __device__ __forceinline__ void store8(float* p, const float* v) {
+  __builtin_nontemporal_store(f32x4{v[0], v[1], v[2], v[3]}, reinterpret_cast<f32x4*>(p));
+  __builtin_nontemporal_store(f32x4{v[4], v[5], v[6], v[7]}, reinterpret_cast<f32x4*>(p + 4));
+}
+// split-K partial tiles are read back by the reduction kernel right away: they stay cacheable
+__device__ __forceinline__ void store8_cached(float* p, const float* v) {
   *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]};
   *reinterpret_cast<f32x4*>(p + 4) = f32x4{v[4], v[5], v[6], v[7]};
+}
+template <typename T>
+__device__ __forceinline__ T __attribute__((ext_vector_type(8))) load8_stream(const void* p) {
+  typedef T raw8 __attribute__((ext_vector_type(8)));
+  if constexpr (sizeof(T) == 2) {
+    return __builtin_bit_cast(raw8, __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p)));
+  } else {
+    raw8 r;
+    const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
+    const f32x4 b = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p) + 1);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      r[e] = a[e];
+      r[4 + e] = b[e];
+    }
+    return r;
+  }
 }
 
 // Stage one operand tile (ROWS rows of the output dimension x BK of the contraction) global -> registers -> LDS.
@@ -249,9 +275,11 @@ __device__ __forceinline__ float frag_f32(const float* lds, int row, int k) {
 // FULL: all 8 columns exist and every pointer allows 16-byte accesses (compile-time trip counts, vector memory
 // operations); otherwise a scalar path bounded by the matrix edge.
 // PRE: the epilogue's per-element inputs (residual / saved activations) were fetched earlier into pre[0..1].
+// hb / hb2: the 8 bias values of columns n .. n+7, already in registers (null: loaded here)
 template <typename T, typename TO, int EPI, bool FULL, bool PRE = false>
 __device__ __forceinline__ void emit8_impl(const GemmParams& p, int64_t m, int64_t n, float* v, const float* u,
-                                           const T __attribute__((ext_vector_type(8))) * pre, float (&cs)[16], bool do_cs) {
+                                           const T __attribute__((ext_vector_type(8))) * pre, float (&cs)[16], bool do_cs,
+                                           const float* hb = nullptr, const float* hb2 = nullptr) {
   TO* Cp = static_cast<TO*>(p.C);
   const T* Rp = static_cast<const T*>(p.R);
   T* auxp = static_cast<T*>(p.aux);
@@ -261,7 +289,9 @@ __device__ __forceinline__ void emit8_impl(const GemmParams& p, int64_t m, int64
   constexpr bool vec = FULL;
 
   if constexpr (EPI == MVIT_EPI_BIAS || EPI == MVIT_EPI_BIAS_RES || EPI == MVIT_EPI_BIAS_GELU || EPI == MVIT_EPI_SWIGLU) {
-    if (bias) {
+    if (hb) {
+      for (int e = 0; e < 8; ++e) v[e] += hb[e];
+    } else if (bias) {
       float b[8];
       if (vec) load8(bias + n, b);
       else
@@ -272,7 +302,9 @@ __device__ __forceinline__ void emit8_impl(const GemmParams& p, int64_t m, int64
   if constexpr (EPI == MVIT_EPI_SWIGLU) {
     float uu[8], h[8];
     for (int e = 0; e < 8; ++e) uu[e] = u[e];
-    if (bias2) {
+    if (hb2) {
+      for (int e = 0; e < 8; ++e) uu[e] += hb2[e];
+    } else if (bias2) {
       float b[8];
       if (vec) load8(bias2 + n, b);
       else
@@ -410,15 +442,16 @@ struct EpiPre {
   }
   // Item `it` of pass a is tile row (RPI*it/32)*WM + a*32 + (RPI*it)%32 + threadIdx/GROUPS: a uniform row offset
   // (scalar address arithmetic) plus the per-thread offset.
+  __device__ __forceinline__ void load_item(const GemmParams& p, int a, int it, raw8 (&dst)[NLOAD]) const {
+    const int rowoff = (RPI * it / 32) * WM + a * 32 + (RPI * it) % 32;
+    const char* r = base + (int64_t)rowoff * p.ldr * (int64_t)sizeof(T);
+    dst[0] = load8_stream<T>(r + thread_off);
+    if (NLOAD == 2) dst[1] = load8_stream<T>(r + p.aux_off * (int64_t)sizeof(T) + thread_off);
+  }
   template <int BUF>
   __device__ __forceinline__ void fetch(const GemmParams& p, int a) {
 #pragma unroll
-    for (int it = 0; it < ITEMS; ++it) {
-      const int rowoff = (RPI * it / 32) * WM + a * 32 + (RPI * it) % 32;
-      const char* r = base + (int64_t)rowoff * p.ldr * (int64_t)sizeof(T);
-      pre[BUF][it][0] = *reinterpret_cast<const raw8*>(r + thread_off);
-      if (NLOAD == 2) pre[BUF][it][1] = *reinterpret_cast<const raw8*>(r + p.aux_off * (int64_t)sizeof(T) + thread_off);
-    }
+    for (int it = 0; it < ITEMS; ++it) load_item(p, a, it, pre[BUF][it]);
   }
 };
 
@@ -483,6 +516,19 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
     if (interior) {
       constexpr int ITEMS = PASS_ROWS * GROUPS / NTHREADS;
       constexpr int NBUF = EP::NBUF;
+      // a thread's items all lie in one 8-column group (NTHREADS is a multiple of GROUPS): its bias values are loaded
+      // once per tile, before the accumulators are parked, instead of once per item behind the previous items' stores
+      // (memory instructions of a wave complete in order, so a load issued after a store also waits for that store)
+      constexpr bool HAS_BIAS = EPI == MVIT_EPI_BIAS || EPI == MVIT_EPI_BIAS_RES || EPI == MVIT_EPI_BIAS_GELU || EPI == MVIT_EPI_SWIGLU;
+      static_assert(NTHREADS % GROUPS == 0, "a thread's items share their column group");
+      float hb[8], hb2[8];
+      if constexpr (HAS_BIAS) {
+        const int64_t nb = n0 + (threadIdx.x % GROUPS) * 8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) hb[e] = hb2[e] = 0.f;
+        if (p.bias) load8(static_cast<const T*>(p.bias) + nb, hb);
+        if (DUAL && p.bias2) load8(static_cast<const T*>(p.bias2) + nb, hb2);
+      }
       if constexpr (EP::HAS_IN) {
         ep.template fetch<0>(p, 0);
         if (NBUF == 2 && MT > 1) ep.template fetch<(NBUF - 1)>(p, 1);
@@ -525,15 +571,19 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
               u[4 + e] = u1[e];
             }
           }
-          if (to_ws) store8(ws + m * p.N + n, v);
-          else if constexpr (EP::HAS_IN) emit8_impl<T, TO, EPI, true, true>(p, m, n, v, u, ep.pre[a % NBUF][it], cs_acc, do_cs);
-          else emit8_impl<T, TO, EPI, true, false>(p, m, n, v, u, nullptr, cs_acc, false);
-        }
-        if constexpr (EP::HAS_IN) {
-          if (a + NBUF < MT) {
-            if ((a % NBUF) == 1) ep.template fetch<(NBUF - 1)>(p, a + NBUF);
-            else ep.template fetch<0>(p, a + NBUF);
-          }
+          if (to_ws) store8_cached(ws + m * p.N + n, v);
+          else if constexpr (EP::HAS_IN) {
+            // the same item of pass a + NBUF is requested before this item's stores are issued: a wave's memory
+            // instructions complete in order, so the wait for a load also waits for every store issued before it
+            typename EP::raw8 nx[EP::NLOAD];
+            if (a + NBUF < MT) ep.load_item(p, a + NBUF, it, nx);
+            emit8_impl<T, TO, EPI, true, true>(p, m, n, v, u, ep.pre[a % NBUF][it], cs_acc, do_cs, HAS_BIAS ? hb : nullptr, nullptr);
+            if (a + NBUF < MT) {
+#pragma unroll
+              for (int k = 0; k < EP::NLOAD; ++k) ep.pre[a % NBUF][it][k] = nx[k];
+            }
+            if constexpr (EP::NLOAD == 2) __builtin_amdgcn_sched_barrier(0);  // keeps the items apart: registers
+          } else emit8_impl<T, TO, EPI, true, false>(p, m, n, v, u, nullptr, cs_acc, false, HAS_BIAS ? hb : nullptr, (HAS_BIAS && DUAL) ? hb2 : nullptr);
         }
       }
       finish_colsum();
@@ -585,7 +635,7 @@ __device__ __forceinline__ void run_epilogue(const GemmParams& p, f32x16 (&acc)[
       }
       if (to_ws) {
         float* w = ws + m * p.N + n;
-        if (ws_vec && n + 8 <= p.N) store8(w, v);
+        if (ws_vec && n + 8 <= p.N) store8_cached(w, v);
         else
           for (int e = 0; e < 8 && n + e < p.N; ++e) w[e] = v[e];
       } else {
