@@ -516,6 +516,13 @@ __device__ __forceinline__ void mfma32x32_init(f32x16& d, const bf16x8& a, const
 __device__ __forceinline__ void mfma32x32_acc(f32x16& d, const bf16x8& a, const u32x4& b) {
   asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(__builtin_bit_cast(u32x4, a)), "a"(b));
 }
+// the same two with both operands in ordinary vector registers
+__device__ __forceinline__ void mfma32x32_init_v(f32x16& d, const bf16x8& a, const bf16x8& b, const f32x16& c) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(__builtin_bit_cast(u32x4, a)), "v"(__builtin_bit_cast(u32x4, b)), "v"(c));
+}
+__device__ __forceinline__ void mfma32x32_acc_v(f32x16& d, const bf16x8& a, const bf16x8& b) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(__builtin_bit_cast(u32x4, a)), "v"(__builtin_bit_cast(u32x4, b)));
+}
 // Moves a fragment into accumulation registers through the lane's own 16-byte LDS slot (a DS load can target them).
 __device__ __forceinline__ u32x4 to_acc_regs(const bf16x8& v, float* slot) {
   const unsigned addr = (unsigned)(uintptr_t)slot;
@@ -1113,6 +1120,275 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
         *reinterpret_cast<bf16x4*>(DK + (int64_t)ki * p.dk_stride + 16 * d + 4 * G4) = a;
         *reinterpret_cast<bf16x4*>(DV + (int64_t)ki * p.dv_stride + 16 * d + 4 * G4) = b;
       }
+    }
+  }
+}
+
+// ================================================================================================
+// Forward for long segments on v_mfma_f32_32x32x16_bf16 only.  A wave owns two blocks of 32 queries (the N dimension of
+// every product), eight waves = 512 queries per work-group, one work-group per CU (two waves per SIMD, ~250 registers).
+// Per tile of 32 keys and query block:
+//   S^T = K Q'^T          5 MFMAs, head_dim contracted exactly; A = a row fragment of the K tile, B = Q' in registers
+//                         the accumulator input is a tile of -m (the running stabiliser), so scores arrive stabilised
+//   P^T = exp2(S^T)       the accumulator layout (lane: query l%32; register i: key 8*(i/4) + 4*(l/32) + i%4) is, after
+//                         packing pairs, already the B operand of the next product: registers 0-7 are contraction
+//                         step 0 (keys 0-15), registers 8-15 step 1, with contraction slot j of lane half hh standing
+//                         for key 16*ks + 4*hh + (j < 4 ? j : j + 4); no lane exchange is needed
+//   O^T += V^T P^T        6 MFMAs: head_dim padded to 96 rows (three 32-row blocks).  Columns 80-95 of the V tile in LDS
+//                         hold ones, so rows 80-95 of O^T accumulate the row sums of P for free.
+// The transposed left factor V^T is read from the natural [key][head_dim] tile with the transposing LDS load using the
+// same slot -> key map.  K / V tiles reach a four-slot LDS ring by direct global -> LDS loads three tiles ahead; lanes
+// that would fill the padding chunks are switched off, so the ones written once at the start stay in place.
+// 16-byte chunk c of row r of a tile sits in slot c ^ xs16(r): sixteen consecutive rows put one chunk index into sixteen
+// different slots (row fragments), four consecutive rows put a pair of chunks into four different 32-byte windows
+// (transposing reads).
+__device__ __forceinline__ int xs16(int row) { return ((row & 3) << 1) | ((row >> 2) & 1) | (((row >> 3) & 1) << 3); }
+__device__ __forceinline__ f32x16 mfma32x32(const bf16x8& a, const bf16x8& b, const f32x16& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+// v_max3_f32 / v_max_f32 as they are: the compiler's fmaxf first quiets a possible signalling NaN in every operand
+// (one more instruction each); scores are finite or -inf
+__device__ __forceinline__ float raw_max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+__device__ __forceinline__ float raw_max(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+// the full maximum of a value held by lanes l and l ^ 32 (the two halves hold different keys of the same query)
+__device__ __forceinline__ float max_across_halves(float x) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));  // a = low half's value, b = high half's, in every lane
+  return raw_max(a, b);
+}
+
+template <int ND>
+__global__ __launch_bounds__(512, 1) void attn_fwd_x32(const AttnParams p) {
+  static_assert(ND == 5, "the padded third block of head_dim and its ones columns are laid out for head_dim 80");
+  using G = Geo<ND>;
+  constexpr int HD = G::HD, BK = 32, RING = 4, QB = 2, WQ = 32 * QB;  // QB blocks of 32 queries per wave
+  constexpr float TAU = 2.f;  // the stabiliser only moves when a score exceeds it by more than TAU (log2 units)
+  __shared__ __attribute__((aligned(1024))) bf16_t lds_k[RING][XS_TILE];
+  __shared__ __attribute__((aligned(1024))) bf16_t lds_v[RING][XS_TILE];
+
+  int seg, h;
+  seg_and_head(p, seg, h);
+  const int s0 = p.cu[seg], L = p.cu[seg + 1] - s0;
+  const int blk_q0 = blockIdx.x * (8 * WQ);
+  if (blk_q0 >= L) return;
+  const int l = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), hh = l >> 5, c32 = l & 31, G4 = l >> 4, r = l & 15;
+  const int q_first = blk_q0 + wv * WQ + c32;  // block qb: query q_first + 32 * qb
+
+  const bf16_t* Q = static_cast<const bf16_t*>(p.q) + (int64_t)s0 * p.q_stride + (int64_t)h * HD;
+  const bf16_t* K = static_cast<const bf16_t*>(p.k) + (int64_t)s0 * p.k_stride + (int64_t)h * HD;
+  const bf16_t* V = static_cast<const bf16_t*>(p.v) + (int64_t)s0 * p.v_stride + (int64_t)h * HD;
+
+  // ones in chunks 10 and 11 (head_dim 80 .. 95) of every row of every V slot
+  for (int i = threadIdx.x; i < RING * 32 * 2; i += 512) {
+    const int slot = i >> 6, row = (i >> 1) & 31, ch = 10 + (i & 1);  // i < RING * 64
+    bf16x8 ones;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ones[j] = (bf16_t)1.f;
+    *reinterpret_cast<bf16x8*>(&lds_v[slot][row * XS_PITCH + ((ch ^ xs16(row)) << 3)]) = ones;
+  }
+
+  // B operand of the score product: Q * scale * log2(e), rounded to bf16 (scores then come out in log2 units)
+  bf16x8 qf[QB][ND];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+    for (int s = 0; s < ND; ++s) {
+      const int qi = q_first + 32 * qb;
+      qf[qb][s] = scale_frag(load_frag_global(Q + (int64_t)qi * p.q_stride + 16 * s + 8 * hh, qi < L), p.scale * LOG2E);
+    }
+
+  // direct global -> LDS loads: one 1 KiB instruction per wave, tensor and tile (rows 4*wv .. 4*wv + 3)
+  const int trow = 4 * wv + (l >> 4);
+  const int tchunk = (l & 15) ^ xs16(trow);
+  const bool tactive = tchunk < 2 * ND;
+  const unsigned lds_k0 = (unsigned)(uintptr_t)&lds_k[0][0], lds_v0 = (unsigned)(uintptr_t)&lds_v[0][0];
+  auto request_tile = [&](int ks, int slot) {
+    if (ks >= L) return;
+    const int row = min(trow, L - 1 - ks);  // rows past the segment end repeat its last row; their scores are masked
+    const unsigned vk = (unsigned)(row * (int)p.k_stride * 2 + tchunk * 16), vv = (unsigned)(row * (int)p.v_stride * 2 + tchunk * 16);
+    if (tactive) {
+      lds_direct_16(lds_k0 + slot * (XS_TILE * 2) + wv * 1024, vk, K + (int64_t)ks * p.k_stride);
+      lds_direct_16(lds_v0 + slot * (XS_TILE * 2) + wv * 1024, vv, V + (int64_t)ks * p.v_stride);
+    }
+  };
+  request_tile(0, 0);
+  request_tile(BK, 1);
+  request_tile(2 * BK, 2);
+  wait_vmcnt<0>();
+  __syncthreads();
+
+  f32x16 o[QB][3];  // O^T: block mt, register i = head_dim 32*mt + 8*(i/4) + 4*hh + i%4 of query l%32; rows 80-95 = row sum of P
+  float m_run[QB];
+  f32x16 negm[QB];  // - m_run in every register: the accumulator input of the score product, so that scores arrive stabilised
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    m_run[qb] = 0.f;
+    negm[qb] = splat16(0.f);
+#pragma unroll
+    for (int mt = 0; mt < 3; ++mt) o[qb][mt] = splat16(0.f);
+  }
+
+  // V^T fragment (block mt of head_dim, contraction step ks): lane i of 16-lane group g4 supplies four consecutive
+  // head-dim values of one key row; the transposing load hands lane j of the group head_dim 32*mt + 16*(g4 & 1) + j
+  // for the four keys 16*ks + 4*(g4 >> 1) + {0..3}, a second load the keys 8 further on
+  auto vt_frag = [&](const bf16_t* tile, int mt, int ks) {
+    const int row = 16 * ks + 4 * (G4 >> 1) + (r >> 2);
+    const int ch = 4 * mt + 2 * (G4 & 1) + ((r & 3) >> 1);
+    const bf16_t* a0 = tile + row * XS_PITCH + ((ch ^ xs16(row)) << 3) + 4 * (r & 1);
+    const bf16_t* a1 = tile + (row + 8) * XS_PITCH + ((ch ^ xs16(row + 8)) << 3) + 4 * (r & 1);
+    return tr_pair(a0, a1);
+  };
+
+  // K row fragments (A operand of the score product) are fetched one tile ahead: tile it+1 is complete in LDS from the
+  // start of iteration it on (see the wait before the barrier), so its fragments are requested under the last MFMAs of
+  // tile it and no LDS latency opens the next iteration
+  bf16x8 kf[ND];
+  auto fetch_k = [&](int slot) {
+#pragma unroll
+    for (int s = 0; s < ND; ++s) kf[s] = *reinterpret_cast<const bf16x8*>(lds_k[slot] + c32 * XS_PITCH + (((2 * s + hh) ^ xs16(c32)) << 3));
+  };
+  fetch_k(0);
+  int it = 0;
+  for (int k0 = 0; k0 < L; k0 += BK, ++it) {
+    const int b0 = it & (RING - 1), b1 = (it + 1) & (RING - 1), b3 = (it + 3) & (RING - 1);
+    request_tile(k0 + 3 * BK, b3);
+    const bf16_t* tv = lds_v[b0];
+    f32x16 sc[QB];
+    unsigned pw[QB][8];
+    auto mask_tail = [&](int qb) {
+      if (k0 + BK > L) {  // last, partial tile
+        asm volatile("" ::: "memory");
+        const int valid = L - k0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (4 * hh >= valid - (8 * (i >> 2) + (i & 3))) sc[qb][i] = -INFINITY;  // key 8*(i/4) + 4*hh + i%4 >= valid
+      }
+    };
+    auto row_max = [&](int qb) {
+      float mx = raw_max3(sc[qb][0], sc[qb][1], sc[qb][2]);
+#pragma unroll
+      for (int i = 3; i < 15; i += 2) mx = raw_max3(mx, sc[qb][i], sc[qb][i + 1]);
+      mx = raw_max(mx, sc[qb][15]);
+      return max_across_halves(mx);
+    };
+    // mx = the largest score of the tile minus the current stabiliser; the stabiliser moves when that excess is above
+    // TAU for some query of the wave (rare after the first tiles): accumulators and this tile's scores are rebased
+    auto rescale = [&](int qb, float mx) {
+      const bool grow = k0 == 0 || mx > TAU;
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+        asm volatile("" ::: "memory");
+        const float delta = grow ? mx : 0.f;
+        const float alpha = k0 == 0 ? 1.f : __builtin_amdgcn_exp2f(-delta);
+        m_run[qb] += delta;
+        negm[qb] = splat16(-m_run[qb]);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sc[qb][i] -= delta;
+#pragma unroll
+        for (int mt = 0; mt < 3; ++mt) o[qb][mt] *= alpha;
+      }
+    };
+    auto p_operand = [&](int qb, int ks) {
+      const u32x4 w4 = {pw[qb][4 * ks], pw[qb][4 * ks + 1], pw[qb][4 * ks + 2], pw[qb][4 * ks + 3]};
+      return __builtin_bit_cast(bf16x8, w4);
+    };
+    {
+      // Two query blocks per wave, software-pipelined by hand: the second block's score MFMAs run under the first
+      // block's softmax arithmetic, the first block's P.V MFMAs under the second block's; scheduling barriers pin the
+      // order.  Only the first score MFMA of each block is inline assembly (its accumulator input is the stabiliser
+      // tile, which the compiler's own MFMA selection would first copy into the result registers).  The compiler sees
+      // no MFMA there and inserts no wait states for its result: the two are issued together, so that a whole MFMA
+      // separates each from the accumulating MFMA that reads its result; all later dependencies are the compiler's.
+      auto words = [&](int qb, int w0, int w1) {
+#pragma unroll
+        for (int w = w0; w < w1; ++w) pw[qb][w] = pack2(__builtin_amdgcn_exp2f(sc[qb][2 * w]), __builtin_amdgcn_exp2f(sc[qb][2 * w + 1]));
+      };
+      mfma32x32_init_v(sc[0], kf[0], qf[0][0], negm[0]);
+      mfma32x32_init_v(sc[1], kf[0], qf[1][0], negm[1]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 1; s < ND; ++s) sc[0] = mfma32x32(kf[s], qf[0][s], sc[0]);
+      sc[1] = mfma32x32(kf[1], qf[1][1], sc[1]);
+      __builtin_amdgcn_sched_barrier(0);
+      mask_tail(0);
+      const float mx0 = row_max(0);
+      rescale(0, mx0);
+      __builtin_amdgcn_sched_barrier(0);
+      sc[1] = mfma32x32(kf[2], qf[1][2], sc[1]);
+      __builtin_amdgcn_sched_barrier(0);
+      words(0, 0, 3);
+      __builtin_amdgcn_sched_barrier(0);
+      sc[1] = mfma32x32(kf[3], qf[1][3], sc[1]);
+      __builtin_amdgcn_sched_barrier(0);
+      words(0, 3, 6);
+      __builtin_amdgcn_sched_barrier(0);
+      sc[1] = mfma32x32(kf[4], qf[1][4], sc[1]);
+      __builtin_amdgcn_sched_barrier(0);
+      words(0, 6, 8);
+      // the V fragments (kept for both blocks) and the first two P.V MFMAs of block 0 separate the last score MFMA of
+      // block 1 from the first read of its result
+      bf16x8 vf[6];
+#pragma unroll
+      for (int n = 0; n < 6; ++n) vf[n] = vt_frag(tv, n % 3, n / 3);
+      o[0][0] = mfma32x32(vf[0], p_operand(0, 0), o[0][0]);
+      o[0][1] = mfma32x32(vf[1], p_operand(0, 0), o[0][1]);
+      __builtin_amdgcn_sched_barrier(0);
+      mask_tail(1);
+      const float mx1 = row_max(1);
+      rescale(1, mx1);
+      __builtin_amdgcn_sched_barrier(0);
+      o[0][2] = mfma32x32(vf[2], p_operand(0, 0), o[0][2]);
+      __builtin_amdgcn_sched_barrier(0);
+      words(1, 0, 2);
+      __builtin_amdgcn_sched_barrier(0);
+      o[0][0] = mfma32x32(vf[3], p_operand(0, 1), o[0][0]);
+      __builtin_amdgcn_sched_barrier(0);
+      words(1, 2, 4);
+      __builtin_amdgcn_sched_barrier(0);
+      o[0][1] = mfma32x32(vf[4], p_operand(0, 1), o[0][1]);
+      __builtin_amdgcn_sched_barrier(0);
+      words(1, 4, 6);
+      __builtin_amdgcn_sched_barrier(0);
+      o[0][2] = mfma32x32(vf[5], p_operand(0, 1), o[0][2]);
+      __builtin_amdgcn_sched_barrier(0);
+      words(1, 6, 8);
+      __builtin_amdgcn_sched_barrier(0);
+      fetch_k(b1);  // next tile's K fragments (garbage past the last tile, never used)
+#pragma unroll
+      for (int n = 0; n < 6; ++n) o[1][n % 3] = mfma32x32(vf[n], p_operand(1, n / 3), o[1][n % 3]);
+    }
+    // tile it+2 (requested one iteration ago) must have landed before any wave reads it; this iteration's own two
+    // requests may stay in flight
+    if (k0 + 3 * BK < L) wait_vmcnt<2>();
+    else wait_vmcnt<0>();
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    const int qi = q_first + 32 * qb;
+    if (qi < L) {
+      const float lsum = o[qb][2][8];  // head_dim row 80 (or 84): the row sum of P
+      const float inv = 1.f / lsum;
+      bf16_t* O = static_cast<bf16_t*>(p.out) + (int64_t)(s0 + qi) * p.o_stride + (int64_t)h * HD;
+#pragma unroll
+      for (int mt = 0; mt < 3; ++mt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (32 * mt + 8 * j >= HD) continue;
+          bf16x4 ov;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) ov[i] = (bf16_t)(o[qb][mt][4 * j + i] * inv);
+          *reinterpret_cast<bf16x4*>(O + 32 * mt + 8 * j + 4 * hh) = ov;
+        }
+      if (hh == 0) p.lse[(int64_t)h * p.total + s0 + qi] = (m_run[qb] + __builtin_amdgcn_logf(lsum)) * LN2;
     }
   }
 }
@@ -1864,6 +2140,13 @@ int launch_fwd_mfma(const AttnParams& p, int n_seg, int max_seqlen, hipStream_t 
     AttnParams pl = p;
     pl.seg_major = 1;  // n_seg fits gridDim.z: checked at the entry point
     dim3 gl = pl.seg_major ? dim3(grid.x, grid.z, grid.y) : grid;
+    if constexpr (ND == 5) {
+      if (max_seqlen >= WIDE_MIN_SEQLEN) {  // 64 queries per wave, 512 per work-group
+        hipLaunchKernelGGL((attn_fwd_x32<ND>), dim3((unsigned)((max_seqlen + 511) / 512), gl.y, gl.z), 512, 0, s, pl);
+        MVIT_CHECK_LAUNCH("attn_fwd");
+        return MVIT_OK;
+      }
+    }
     hipLaunchKernelGGL((attn_fwd_mfma<ND, 8, 32, true, 2, 4>), gl, 512, 0, s, pl);
   }
   else hipLaunchKernelGGL((attn_fwd_mfma<ND, 4, 32, true>), grid, 256, 0, s, p);  // head_dim 128: register budget
