@@ -116,7 +116,7 @@ KERNEL_NAMES = {
     "gemm_nt_epi5": "gemm_dl_kernel<TO, TA=false, TB=true, EPI=SWIGLU_BWD>",
     "gemm_nt_epi6": "gemm_dl_kernel<TO, TA=false, TB=true, EPI=GELU_BWD>",
     "gemm_tt_epi0": "gemm_dl_kernel<TO, TA=true, TB=true, EPI=NONE, MI16> + splitk_reduce_kernel",
-    "attn_fwd_full": "attn_fwd_mfma<5, 8, 32, true, 2, 4>",
+    "attn_fwd_full": "attn_fwd_x32<5> (segments >= 512 tokens), attn_fwd_mfma<5, 8, 32, true, 2, 4> (shorter)",
     "attn_bwd_full": "attn_delta_rows_kernel + attn_bwd_prepare_kernel + attn_bwd_dkdv_wide<5> + attn_bwd_dq_wide<5>",
     "attn_fwd_window": "attn_fwd_mfma<5, 2, 64, false, 2, 4>",
     "attn_bwd_window": "attn_bwd_window_mfma<5, 4, 2>",
