@@ -29,6 +29,7 @@ for _p in (ROOT, ROOT / "multimodal-training_amd"):
     if str(_p) not in sys.path:
         sys.path.insert(0, str(_p))
 
+import numpy as np  # noqa: E402
 import torch  # noqa: E402
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
@@ -198,14 +199,6 @@ def handoff_leg(n_vision: int, hidden: int, dtype, iters: int = 20):
         text.grad = None
         return extract_vision_grad(leaf)
 
-    def timed(fn):
-        fn()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(iters):
-            fn()
-        torch.cuda.synchronize()
-        return 1000.0 * (time.perf_counter() - t0) / iters
 
     assert torch.equal(ours(), reference_calls())
     ours_ms, ref_ms = timed(ours), timed(reference_calls)
@@ -254,6 +247,26 @@ def input_leg(grid, dtype, iters: int = 20):
         torch.cuda.synchronize()
         return 1000.0 * (time.perf_counter() - t0) / iters
 
+    # the resize in front of it (PIL bicubic, bit-identical on the GPU): the workload's largest image from a decoded
+    # frame 1.25 x its size, against Pillow on one host core (one call, bounded)
+    from mi355_vit.pixels import resize_frames
+
+    big = max(frames, key=lambda f: f.shape[1] * f.shape[2])
+    th, tw = int(big.shape[1]), int(big.shape[2])
+    raw = torch.randint(0, 256, (1, th * 5 // 4, tw * 5 // 4, 3), generator=g, dtype=torch.uint8)
+    raw_dev = raw.to(dev)
+    resize_ms = timed(lambda: resize_frames(raw_dev, th, tw))
+    resize_gbs = (raw.numel() + th * tw * 3) / (resize_ms * 1e-3) / 1e9
+    pil_ms = pil_same = None
+    try:
+        from PIL import Image
+        t0 = time.perf_counter()
+        ref = np.asarray(Image.fromarray(raw[0].numpy()).resize((tw, th), Image.Resampling.BICUBIC))
+        pil_ms = 1000.0 * (time.perf_counter() - t0)
+        pil_same = bool(np.array_equal(resize_frames(raw_dev, th, tw)[0].cpu().numpy(), ref))
+    except ImportError:
+        pass
+
     same = bool(torch.equal(ours(), torch_ops()))  # bit for bit wherever torch's own kernels divide exactly
     max_diff = float((ours().float() - torch_ops().float()).abs().max())
     ours_ms, ref_ms = timed(ours), timed(torch_ops)
@@ -261,7 +274,10 @@ def input_leg(grid, dtype, iters: int = 20):
     moved = frame_bytes + rows * 1176 * out.element_size()  # every input byte once, every output value once
     return {"images": len(frames), "rows": rows, "frame_bytes": frame_bytes, "out_dtype": str(dtype).replace("torch.", ""),
             "patchify_ms": round(ours_ms, 3), "algorithmic_gbs": round(moved / (ours_ms * 1e-3) / 1e9, 1),
-            "torch_ops_ms": round(ref_ms, 3), "equals_torch_ops": same, "max_abs_diff_vs_torch_ops": max_diff}
+            "torch_ops_ms": round(ref_ms, 3), "equals_torch_ops": same, "max_abs_diff_vs_torch_ops": max_diff,
+            "resize": {"from": [int(raw.shape[1]), int(raw.shape[2])], "to": [th, tw], "filter": "bicubic", "gpu_ms": round(resize_ms, 3),
+                       "algorithmic_gbs": round(resize_gbs, 1), "pillow_one_core_ms": None if pil_ms is None else round(pil_ms, 1),
+                       "equals_pillow": pil_same}}
 
 
 def cpu_baseline(cfg_kw, grid, seed, dtype, budget_s: float = 30.0):

@@ -295,6 +295,22 @@ typedef struct mvit_image {
 int mvit_patchify(const mvit_image* images, int n_images, int64_t total_rows, void* out, double rescale, float mean_r,
                   float mean_g, float mean_b, float std_r, float std_g, float std_b, int dtype, mvit_stream_t stream);
 
+/* One resampling pass of PIL.Image.resize for 8-bit images along the middle axis of a contiguous uint8 array
+ * [outer][in_len][inner] -> [outer][out_len][inner] (device memory): for output coordinate x the in-range window of
+ * bounds[2x + 1] input coordinates starting at bounds[2x], weighted by the 22-bit fixed-point coefficients
+ * kk[x * ksize + i]; accumulator = 2^21 + sum byte * weight, result = clamp(accumulator >> 22, 0, 255): Pillow's
+ * libImaging/Resample.c (ImagingResampleHorizontal_8bpc / ImagingResampleVertical_8bpc), bit for bit.  A resize is
+ * the horizontal pass (outer = frames * height, inner = 3) into an intermediate image followed by the vertical pass
+ * (outer = frames, inner = new_width * 3); a pass whose size does not change is skipped by the caller.  bounds and kk
+ * are device arrays that the host computes once per (in_len, out_len, filter) as Resample.c precompute_coeffs +
+ * normalize_coeffs_8bpc do (Python: mi355_vit.pixels.resample_coefficients).
+ * Replaces, for frames that are already on the GPU, the two PIL resizes in front of the patch rows: the reference's
+ * own fixed-size BILINEAR resize (python/data/preprocessing.py:126-131) and the BICUBIC resize to the smart_resize
+ * target inside the image processor (transformers 4.57.0 Qwen2VLImageProcessor, reached through
+ * processor.apply_chat_template, python/data/preprocessing.py:134). */
+int mvit_resample_u8(const uint8_t* src, uint8_t* dst, int64_t outer, int64_t in_len, int64_t out_len, int64_t inner,
+                     const int32_t* bounds, const int32_t* kk, int ksize, mvit_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

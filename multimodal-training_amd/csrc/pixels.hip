@@ -108,6 +108,113 @@ __global__ __launch_bounds__(256) void patchify_kernel(const mvit_image* __restr
 
 }  // namespace
 
+// ------------------------------------------------------------------------------------------------
+// One resampling pass along the middle axis of a uint8 array [outer][in_len][inner] -> [outer][out_len][inner], with
+// Pillow's 8-bit arithmetic (libImaging/Resample.c, ImagingResampleHorizontal_8bpc / Vertical_8bpc): per output
+// coordinate a window of `bounds[2*x + 1]` input coordinates starting at `bounds[2*x]`, 22-bit fixed-point weights
+// kk[x * ksize + i], an accumulator that starts at one half, an arithmetic shift and a clamp to 0..255.
+// A thread makes four consecutive output bytes of one output coordinate (inner is the contiguous dimension: pixels
+// times channels for the vertical pass, 3 channels for the horizontal one) or, when inner is not a multiple of four,
+// four consecutive bytes of the flattened [out_len * inner] row, each with its own window.
+constexpr int RESAMPLE_PRECISION_BITS = 22;
+__device__ __forceinline__ unsigned clip8(int v) {
+  v >>= RESAMPLE_PRECISION_BITS;
+  return (unsigned)(v < 0 ? 0 : (v > 255 ? 255 : v));
+}
+template <bool WIDE>  // WIDE: inner % 4 == 0 and 4-byte aligned rows, the four bytes share one window
+__global__ __launch_bounds__(256) void resample_pass_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int64_t outer,
+                                                            int64_t in_len, int64_t out_len, int64_t inner,
+                                                            const int32_t* __restrict__ bounds, const int32_t* __restrict__ kk, int ksize) {
+  const int64_t row_out = out_len * inner, row_in = in_len * inner;
+  const int64_t quads = (row_out + 3) / 4;
+  const int64_t total = outer * quads;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t o = i / quads, q = i % quads;
+    const uint8_t* s = src + o * row_in;
+    uint8_t* d = dst + o * row_out + 4 * q;
+    if (WIDE) {
+      const int64_t x = (4 * q) / inner, c = (4 * q) % inner;
+      const int xmin = bounds[2 * x], n = bounds[2 * x + 1];
+      const int32_t* k = kk + x * ksize;
+      int a0 = 1 << (RESAMPLE_PRECISION_BITS - 1), a1 = a0, a2 = a0, a3 = a0;
+      for (int t = 0; t < n; ++t) {
+        const unsigned w = *reinterpret_cast<const unsigned*>(s + (int64_t)(xmin + t) * inner + c);
+        const int kt = k[t];
+        a0 += (int)(w & 0xff) * kt;
+        a1 += (int)((w >> 8) & 0xff) * kt;
+        a2 += (int)((w >> 16) & 0xff) * kt;
+        a3 += (int)(w >> 24) * kt;
+      }
+      *reinterpret_cast<unsigned*>(d) = clip8(a0) | (clip8(a1) << 8) | (clip8(a2) << 16) | (clip8(a3) << 24);
+    } else {
+      for (int b = 0; b < 4; ++b) {
+        const int64_t e = 4 * q + b;
+        if (e >= row_out) break;
+        const int64_t x = e / inner, c = e % inner;
+        const int xmin = bounds[2 * x], n = bounds[2 * x + 1];
+        const int32_t* k = kk + x * ksize;
+        int a = 1 << (RESAMPLE_PRECISION_BITS - 1);
+        for (int t = 0; t < n; ++t) a += (int)s[(int64_t)(xmin + t) * inner + c] * k[t];
+        d[b] = (uint8_t)clip8(a);
+      }
+    }
+  }
+}
+
+// The same pass for a short contiguous dimension (the horizontal pass: inner = channels): neighbouring output bytes have
+// different windows and every tap is a single byte, so a work-group first copies its input row into LDS with aligned
+// 4-byte loads and then reads the taps from there.  One work-group per row of the outer dimension; a thread makes whole
+// pixels (up to four channels).
+constexpr int RESAMPLE_LDS_BYTES = 60 * 1024, RESAMPLE_MAX_CHANNELS = 4;
+__global__ __launch_bounds__(256) void resample_rows_lds_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int64_t outer,
+                                                                int64_t in_len, int64_t out_len, int inner,
+                                                                const int32_t* __restrict__ bounds, const int32_t* __restrict__ kk, int ksize) {
+  __shared__ __attribute__((aligned(16))) uint8_t row[RESAMPLE_LDS_BYTES + 8];
+  const int64_t row_in = in_len * inner, row_out = out_len * inner;
+  const uint8_t* src_end = src + outer * row_in;
+  for (int64_t o = blockIdx.x; o < outer; o += gridDim.x) {
+    const uint8_t* b = src + o * row_in;
+    const int lead = (int)((uintptr_t)b & 3);  // the row starts `lead` bytes into an aligned word
+    const uint8_t* a = b - lead;
+    const int words = (int)((lead + row_in + 3) / 4);
+    __syncthreads();  // the previous row has been consumed
+    for (int j = threadIdx.x; j < words; j += 256) {
+      const uint8_t* g = a + 4 * j;
+      unsigned w;
+      if (g >= src && g + 4 <= src_end) {
+        w = *reinterpret_cast<const unsigned*>(g);
+      } else {  // first / last word of the array: only the bytes that belong to it
+        w = 0;
+        for (int e = 0; e < 4; ++e)
+          if (g + e >= src && g + e < src_end) w |= (unsigned)g[e] << (8 * e);
+      }
+      *reinterpret_cast<unsigned*>(row + 4 * j) = w;
+    }
+    __syncthreads();
+    const uint8_t* r = row + lead;
+    uint8_t* d = dst + o * row_out;
+    // a thread makes whole pixels: the channels of a pixel share its window and its weights
+    for (int x = threadIdx.x; x < (int)out_len; x += 256) {
+      const int xmin = bounds[2 * x], n = bounds[2 * x + 1];
+      const int32_t* k = kk + (int64_t)x * ksize;
+      int acc[RESAMPLE_MAX_CHANNELS];
+#pragma unroll
+      for (int c = 0; c < RESAMPLE_MAX_CHANNELS; ++c) acc[c] = 1 << (RESAMPLE_PRECISION_BITS - 1);
+      const uint8_t* px = r + xmin * inner;
+      for (int t = 0; t < n; ++t) {
+        const int kt = k[t];
+#pragma unroll
+        for (int c = 0; c < RESAMPLE_MAX_CHANNELS; ++c)
+          if (c < inner) acc[c] += (int)px[c] * kt;
+        px += inner;
+      }
+#pragma unroll
+      for (int c = 0; c < RESAMPLE_MAX_CHANNELS; ++c)
+        if (c < inner) d[x * inner + c] = (uint8_t)clip8(acc[c]);
+    }
+  }
+}
+
 extern "C" {
 
 int mvit_patchify(const mvit_image* images, int n_images, int64_t total_rows, void* out, double rescale, float mean_r,
@@ -127,6 +234,26 @@ int mvit_patchify(const mvit_image* images, int n_images, int64_t total_rows, vo
   else
     hipLaunchKernelGGL((patchify_kernel<float>), dim3(grid), 256, 0, s, images, n_images, static_cast<float*>(out), total_rows, nm);
   MVIT_CHECK_LAUNCH("patchify");
+  return MVIT_OK;
+}
+
+int mvit_resample_u8(const uint8_t* src, uint8_t* dst, int64_t outer, int64_t in_len, int64_t out_len, int64_t inner,
+                     const int32_t* bounds, const int32_t* kk, int ksize, mvit_stream_t stream) {
+  MVIT_REQUIRE(src && dst && bounds && kk, "resample_u8: null pointer");
+  MVIT_REQUIRE(outer >= 0 && in_len > 0 && out_len > 0 && inner > 0 && ksize > 0, "resample_u8: bad sizes (outer=%lld in=%lld out=%lld inner=%lld ksize=%d)",
+               (long long)outer, (long long)in_len, (long long)out_len, (long long)inner, ksize);
+  MVIT_REQUIRE(in_len < (1 << 24) && out_len < (1 << 24) && in_len * inner < (1ll << 40) && out_len * inner < (1ll << 40), "resample_u8: axis too long");
+  if (outer == 0) return MVIT_OK;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int64_t quads = (out_len * inner + 3) / 4, total = outer * quads;
+  const unsigned grid = (unsigned)((total + 255) / 256 < 65535 * 16 ? (total + 255) / 256 : 65535 * 16);
+  const bool wide = inner % 4 == 0 && ((uintptr_t)src % 4 == 0) && ((uintptr_t)dst % 4 == 0);
+  if (!wide && inner <= RESAMPLE_MAX_CHANNELS && in_len * inner + 4 <= RESAMPLE_LDS_BYTES) {
+    const unsigned rows = (unsigned)(outer < 65535 * 16 ? outer : 65535 * 16);
+    hipLaunchKernelGGL(resample_rows_lds_kernel, dim3(rows), 256, 0, s, src, dst, outer, in_len, out_len, (int)inner, bounds, kk, ksize);
+  } else if (wide) hipLaunchKernelGGL((resample_pass_kernel<true>), dim3(grid), 256, 0, s, src, dst, outer, in_len, out_len, inner, bounds, kk, ksize);
+  else hipLaunchKernelGGL((resample_pass_kernel<false>), dim3(grid), 256, 0, s, src, dst, outer, in_len, out_len, inner, bounds, kk, ksize);
+  MVIT_CHECK_LAUNCH("resample_u8");
   return MVIT_OK;
 }
 

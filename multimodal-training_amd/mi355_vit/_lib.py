@@ -78,6 +78,7 @@ PROTOTYPES = {
     "mvit_grad_sumsq": [_vp, _i32, _i64, _vp, _vp, _i32, _vp],
     "mvit_grad_sumsq_static": [_vp, _i32, _i64, _vp, _i32, _vp],
     "mvit_patchify": [_vp, _i32, _i64, _vp, C.c_double] + [_f32] * 6 + [_i32, _vp],
+    "mvit_resample_u8": [_vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _i32, _vp],
     "mvit_attn_bwd": [_vp] * 12 + [_i32, _i32, _i64, _i32, _i32] + [_i64] * 8 + [_f32, _i32, _vp],
 }
 EXPORTS = sorted(list(PROTOTYPES) + ["mvit_version", "mvit_last_error"])

@@ -341,6 +341,18 @@ class BaseVisionTrainer(Trainer):
             sample_index = sample_index.item() if sample_index.numel() == 1 else sample_index.tolist()
         device = torch.device("cuda:0")
         batch = dict(batch)
+        if batch.get("pixel_values") is None and batch.get("frames") is None and batch.get("raw_images") is not None:
+            # decoded still images of any size (uint8 [1, H, W, 3]): the processor's smart_resize + bicubic resize run on
+            # the GPU as well (bit-identical to PIL), then the frames path below
+            from .pixels import resize_frames, smart_resize
+
+            limits = {k: int(self.config[k]) for k in ("min_pixels", "max_pixels") if self.config.get(k) is not None}
+            frames = []
+            for f in batch["raw_images"]:
+                f = f.to(device, non_blocking=True).contiguous()
+                th, tw = smart_resize(int(f.shape[1]), int(f.shape[2]), **limits)
+                frames.append(resize_frames(f, th, tw))
+            batch["frames"] = frames
         if batch.get("pixel_values") is None and batch.get("frames") is not None:
             # resized uint8 frames ([frames, H, W, 3] per image or video) instead of the processor's float rows:
             # a fifth of the upload, and rescale / normalise / patchify run on the GPU in the model's dtype

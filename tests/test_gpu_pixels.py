@@ -155,3 +155,82 @@ def test_patchify_rejects_what_it_cannot_do():
         patchify([])
     with pytest.raises(RuntimeError, match="contiguous"):
         patchify([torch.zeros(1, 28, 56, 3, dtype=torch.uint8, device=DEV)[:, :, ::2]])
+
+
+# ------------------------------------------------------------------------------------------------ resize
+
+
+def _resize_gpu(img, oh, ow, name):
+    from mi355_vit.pixels import resize_frames
+
+    out = resize_frames(torch.from_numpy(img).to(DEV), oh, ow, name)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+@pytest.mark.parametrize("name", ["bilinear", "bicubic"])
+def test_resize_bit_exact_against_oracle_and_pillow(name):
+    """Up- and down-scaling, one pass skipped, videos (several frames), odd widths (the byte-wise path of the vertical
+    pass), against the oracle and, where Pillow is installed, against PIL.Image.resize itself."""
+    from oracle import resize_oracle as ro
+
+    rng = np.random.default_rng(11)
+    cases = [(1, 37, 53, 28, 56), (1, 100, 80, 56, 56), (2, 28, 28, 112, 84), (1, 5, 7, 28, 28), (3, 64, 64, 64, 32), (1, 64, 60, 28, 60),
+             (1, 211, 157, 140, 196), (1, 33, 1, 28, 28), (1, 90, 61, 45, 33), (1, 300, 200, 299, 201)]
+    try:
+        from PIL import Image
+        filt = {"bilinear": Image.Resampling.BILINEAR, "bicubic": Image.Resampling.BICUBIC}[name]
+    except ImportError:
+        Image = None
+    for f, h, w, oh, ow in cases:
+        _announce(f"resize {name} {f}x{h}x{w} -> {oh}x{ow}")
+        img = rng.integers(0, 256, (f, h, w, 3), dtype=np.uint8)
+        got = _resize_gpu(img, oh, ow, name)
+        assert got.shape == (f, oh, ow, 3) and got.dtype == np.uint8
+        for i in range(f):
+            assert np.array_equal(got[i], ro.pil_resize(img[i], oh, ow, name)), (f, h, w, oh, ow, i)
+            if Image is not None:
+                assert np.array_equal(got[i], np.asarray(Image.fromarray(img[i]).resize((ow, oh), filt)))
+
+
+def test_resize_large_image_against_pillow_and_the_whole_input_chain():
+    """A 2,000 x 3,000 photograph-sized image through smart_resize -> bicubic resize -> patchify on the GPU equals the
+    same chain on the CPU (Pillow resize where installed, else the oracle; oracle patchify), bit for bit in float32."""
+    from oracle import resize_oracle as ro
+    from mi355_vit import pixels as P
+
+    _announce("resize 2000x3000 + patchify chain")
+    rng = np.random.default_rng(12)
+    # smooth content plus noise, so that neighbouring pixels are correlated like in a photograph
+    base = rng.integers(0, 256, (1, 50, 75, 3), dtype=np.uint8)
+    big = np.clip(np.kron(base, np.ones((1, 40, 40, 1))) + rng.integers(-20, 21, (1, 2000, 3000, 3)), 0, 255).astype(np.uint8)
+    th, tw = P.smart_resize(2000, 3000)
+    assert (th, tw) == ro.smart_resize(2000, 3000) and th % 28 == 0 and tw % 28 == 0
+    got = _resize_gpu(big, th, tw, "bicubic")
+    try:
+        from PIL import Image
+        ref = np.asarray(Image.fromarray(big[0]).resize((tw, th), Image.Resampling.BICUBIC))[None]
+    except ImportError:
+        ref = ro.pil_resize(big[0], th, tw, "bicubic")[None]
+    assert np.array_equal(got, ref)
+    pv, grid = P.preprocess([torch.from_numpy(big).to(DEV)])
+    torch.cuda.synchronize()
+    ref_pv, ref_grid = po.patchify_batch([ref])
+    assert grid.tolist() == ref_grid.tolist() == [[1, th // 14, tw // 14]]
+    assert np.array_equal(pv.cpu().numpy().view(np.uint32), ref_pv.view(np.uint32))
+
+
+def test_resize_rejects_what_it_cannot_do():
+    from mi355_vit.pixels import resize_frames
+
+    x = torch.zeros(1, 28, 28, 3, dtype=torch.uint8, device=DEV)
+    with pytest.raises(ValueError):
+        resize_frames(x.float(), 28, 28)
+    with pytest.raises(ValueError):
+        resize_frames(x, 0, 28)
+    with pytest.raises(ValueError):
+        resize_frames(x, 28, 56, "lanczos")
+    with pytest.raises(RuntimeError):
+        resize_frames(x.cpu(), 56, 56)
+    same = resize_frames(x, 28, 28)
+    assert same.data_ptr() != x.data_ptr() and torch.equal(same, x)
