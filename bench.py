@@ -216,7 +216,8 @@ def input_leg(grid, dtype, iters: int = 20):
 
     dev = torch.device("cuda:0")
     g = torch.Generator().manual_seed(0)
-    frames = [torch.randint(0, 256, (int(t), 14 * int(h), 14 * int(w), 3), generator=g, dtype=torch.uint8).to(dev)
+    # a grid entry with t = 1 is a still image (one frame fills both halves of a row), t > 1 a video of 2 t frames
+    frames = [torch.randint(0, 256, (1 if t == 1 else 2 * int(t), 14 * int(h), 14 * int(w), 3), generator=g, dtype=torch.uint8).to(dev)
               for t, h, w in grid.tolist()]
     rows = int(grid.prod(dim=1).sum())
     out = torch.empty((rows, 1176), dtype=dtype, device=dev)
@@ -267,6 +268,28 @@ def input_leg(grid, dtype, iters: int = 20):
     except ImportError:
         pass
 
+    # the patch embedding straight from the frames (rows made inside the GEMM) against patchify + GEMM, bf16
+    patch_embed = None
+    if dtype == torch.bfloat16:
+        from mi355_vit import ops
+        from mi355_vit.pixels import pack_patch_embed_weight, patch_embed_frames
+
+        w = (torch.randn(1280, 1176, generator=g) * 0.03).to(dev, torch.bfloat16)
+        two_out = torch.empty((rows, 1280), dtype=dtype, device=dev)
+
+        def fused():
+            return patch_embed_frames(frames, pack_patch_embed_weight(w), dtype=dtype)[0]
+
+        def two_kernels():
+            ops.gemm(patchify(frames, dtype=dtype, out=out)[0], w, two_out)
+            return two_out
+
+        diff = float((fused().float() - two_kernels().float()).abs().max() / two_kernels().float().abs().max())
+        fused_ms, two_ms = timed(fused), timed(two_kernels)
+        patch_embed = {"embed_dim": 1280, "from_frames_ms": round(fused_ms, 3), "patchify_plus_gemm_ms": round(two_ms, 3),
+                       "tflops_counted_on_k_1176": round(2.0 * rows * 1176 * 1280 / (fused_ms * 1e-3) / 1e12, 1),
+                       "max_rel_diff": diff}
+
     same = bool(torch.equal(ours(), torch_ops()))  # bit for bit wherever torch's own kernels divide exactly
     max_diff = float((ours().float() - torch_ops().float()).abs().max())
     ours_ms, ref_ms = timed(ours), timed(torch_ops)
@@ -277,7 +300,8 @@ def input_leg(grid, dtype, iters: int = 20):
             "torch_ops_ms": round(ref_ms, 3), "equals_torch_ops": same, "max_abs_diff_vs_torch_ops": max_diff,
             "resize": {"from": [int(raw.shape[1]), int(raw.shape[2])], "to": [th, tw], "filter": "bicubic", "gpu_ms": round(resize_ms, 3),
                        "algorithmic_gbs": round(resize_gbs, 1), "pillow_one_core_ms": None if pil_ms is None else round(pil_ms, 1),
-                       "equals_pillow": pil_same}}
+                       "equals_pillow": pil_same},
+            "patch_embed": patch_embed}
 
 
 def cpu_baseline(cfg_kw, grid, seed, dtype, budget_s: float = 30.0):
@@ -475,9 +499,12 @@ def main() -> None:
         t = timed_steps(train_step, 1, n)
         return {"steps": n, "ms_per_step": round(1000.0 * t / n, 3), "patches_per_s": round(S / (t / n), 1)}
 
-    def other_workload(name):
-        """Forward + backward of another configuration on the same tower (weights as they are), timing only."""
+    def other_workload(name, checkpointing=None):
+        """Forward + backward of another configuration on the same tower (weights as they are), timing only.
+        ``checkpointing`` overrides the configuration's own setting (None: as the configuration says)."""
         _, _, _, grid2, seed2, ckpt2 = make_workload(name)
+        if checkpointing is not None:
+            ckpt2 = checkpointing
         S2 = int(grid2.prod(dim=1).sum())
         g2 = torch.Generator(device="cpu").manual_seed(seed2)
         px = torch.randn(S2, 1176, generator=g2).to(dev)
@@ -489,17 +516,23 @@ def main() -> None:
             model.zero_grad(set_to_none=True)
             model(hidden_states=px, grid_thw=gd).backward(go)
 
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
         try:
             t = timed_steps(step2, 2, 5)
         finally:
             (model.gradient_checkpointing_enable if ckpt else model.gradient_checkpointing_disable)()
         return {"patches": S2, "grid_thw": grid2.tolist(), "activation_checkpointing": ckpt2, "steps": 5,
-                "ms_per_step": round(1000.0 * t / 5, 3), "patches_per_s": round(S2 / (t / 5), 1)}
+                "ms_per_step": round(1000.0 * t / 5, 3), "patches_per_s": round(S2 / (t / 5), 1),
+                "peak_mem_gb": round(torch.cuda.max_memory_allocated() / 2**30, 2)}
 
     optimizer = handoff = input_side = with_opt = None
     others = None
     if not args.no_other_workloads and cfg_kw == FULL_TOWER:
         others = {name: side_leg(other_workload, name) for name in ("cfg2", "cfg3", "cfg5") if name != args.workload}
+        # the 65,536-patch image with every activation kept (no block is run twice): what 288 GB of HBM allow;
+        # reported beside the metric, which stays on the configuration as it is named (checkpointing per block)
+        others["cfg3_all_activations_kept"] = side_leg(other_workload, "cfg3", False)
     if not args.no_optimizer:
         with_opt = side_leg(with_optimizer_leg)
         optimizer = side_leg(optimizer_leg, model, step)

@@ -295,6 +295,25 @@ typedef struct mvit_image {
 int mvit_patchify(const mvit_image* images, int n_images, int64_t total_rows, void* out, double rescale, float mean_r,
                   float mean_g, float mean_b, float std_r, float std_g, float std_b, int dtype, mvit_stream_t stream);
 
+/* The patch embedding straight from decoded frames: out[r, :] = row r of pixel_values (exactly the bf16 rows that
+ * mvit_patchify makes for the same table and constants) x weight^T, bf16 MFMA with fp32 accumulation, without the
+ * [total_rows, 1176] matrix ever being written.  The kernel contracts along memory (frame of the pair, y | x, channel)
+ * instead of (channel, frame, y, x), so it takes the weight re-ordered by mvit_patch_embed_pack_weight:
+ *   packed[n, (frame * 14 + y) * 48 + x * 3 + channel] = w[n, channel * 392 + frame * 196 + y * 14 + x], zero elsewhere;
+ *   packed is [n_out, 1344] bf16, 16-byte aligned; w is [n_out, >= 1176] of dtype MVIT_BF16 or MVIT_F32, row pitch ldw.
+ * Frame buffers must be 4-byte aligned (their size always is a multiple of 4: widths are multiples of 28); the table
+ * is trusted as in mvit_patchify.  Rescale and normalisation run as one fused multiply-add per byte; constants for
+ * which that does not reproduce mvit_patchify's bf16 values for all 3 x 256 inputs are rejected with
+ * MVIT_ERR_UNSUPPORTED (the caller then uses mvit_patchify + mvit_gemm).  out is [total_rows, ldo >= n_out] of
+ * out_dtype MVIT_BF16 or MVIT_F32.
+ * Replaces the image processor's rescale / normalise / patchify (python/data/preprocessing.py:134) together with the
+ * tower's patch embedding, Qwen2_5_VisionPatchEmbed.forward (python/models/qwen2_5_vl/modeling_qwen2_5_vl.py:225-231:
+ * a Conv3d without bias whose kernel equals its stride, i.e. this matrix product). */
+int mvit_patch_embed_pack_weight(const void* w, int dtype, int64_t ldw, int64_t n_out, void* packed, mvit_stream_t stream);
+int mvit_patch_embed_frames(const mvit_image* images, int n_images, int64_t total_rows, const void* packed_w, int64_t n_out,
+                            void* out, int64_t ldo, int out_dtype, double rescale, float mean_r, float mean_g, float mean_b,
+                            float std_r, float std_g, float std_b, mvit_stream_t stream);
+
 /* One resampling pass of PIL.Image.resize for 8-bit images along the middle axis of a contiguous uint8 array
  * [outer][in_len][inner] -> [outer][out_len][inner] (device memory): for output coordinate x the in-range window of
  * bounds[2x + 1] input coordinates starting at bounds[2x], weighted by the 22-bit fixed-point coefficients

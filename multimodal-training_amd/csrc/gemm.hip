@@ -14,6 +14,8 @@
 // read and results written as 16-byte vectors along N.
 // Work-group ids are remapped so that the tiles a single XCD (one L2) works on are neighbours in N.
 #include "mvit_common.h"
+#include <string.h>
+#include <type_traits>
 
 namespace {
 
@@ -41,6 +43,11 @@ struct GemmParams {
   int vec_ok;         // every epilogue pointer / stride allows 16-byte accesses
   float* colsum;      // SWIGLU_BWD: per-tile-row column sums of the output, [tiles_m][ldc] (null: not wanted)
   int panel_w;        // tiles are walked in panels of this many tile columns (M fastest across a panel's rows)
+  // A operand made from decoded frames (gemm_dl_kernel<..., PIX = true>): image table and the affine form of the
+  // rescale / normalise step, value = byte * px_a[channel] + px_c[channel]
+  const mvit_image* px_images;
+  int px_n_images;
+  float px_a[3], px_c[3];
 };
 
 // Tile order inside one K slice: panels of panel_w tile columns; within a panel row by row.  Work-groups that run
@@ -239,6 +246,75 @@ struct TileLoader {
   }
 };
 
+// The A operand of the patch embedding made on the fly from decoded uint8 frames (no [rows, 1176] matrix in memory).
+// The contraction index is re-ordered so that it runs along memory: k' = line * 48 + b with line = frame-of-the-pair *
+// 14 + y and b = x * 3 + channel for b < 42 (the 42 bytes of one pixel line of a patch are contiguous in the frame);
+// b = 42..47 pads the line to six 8-byte pieces and meets zero weights (mvit_patch_embed_pack_weight).
+// 1344 = 28 lines * 48 = 42 K tiles of 32.  A lane fetches one 8-byte piece per row and K tile with a single vector load
+// and turns it into a 16-byte bf16 chunk with eight conversions byte -> float -> a * x + c -> bf16.  Pieces advance by a
+// fixed count per K tile, so (line, piece) and the channel of the piece's first byte are stepped, not recomputed.
+constexpr int PX_LINE = 48, PX_LINES = 28, PX_K = PX_LINE * PX_LINES, PX_PATCH = 14;
+__device__ __forceinline__ int px_find_image(const mvit_image* t, int n, int64_t row) {
+  int lo = 0, hi = n;  // invariant: t[lo].first_row <= row < t[hi].first_row
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (t[mid].first_row <= row) lo = mid;
+    else hi = mid;
+  }
+  return lo;
+}
+// Where patch `row` of the batch lies: first byte of its 14 x 14 pixel square in the first frame of its temporal pair,
+// bytes per image line, distance to the pair's second frame (0 when
+// the last frame of an odd count, or a still image, fills both halves).
+__device__ __forceinline__ void px_locate(const GemmParams& p, int64_t row, const uint8_t*& base, int& line_bytes, int& frame_off) {
+  if (row >= p.M) row = p.M - 1;  // rows past the edge repeat the last row; their results are never stored
+  const mvit_image im = p.px_images[px_find_image(p.px_images, p.px_n_images, row)];
+  const int gh = im.height / PX_PATCH, gw = im.width / PX_PATCH, per_t = gh * gw;
+  const int64_t local = row - im.first_row;
+  const int t = (int)(local / per_t), rem = (int)(local % per_t);
+  // rem = ((block row * (gw / 2) + block column) * 2 + row in block) * 2 + column in block
+  const int blk = rem >> 2, hb = blk / (gw >> 1), wb = blk % (gw >> 1);
+  const int y0 = (2 * hb + ((rem >> 1) & 1)) * PX_PATCH, x0 = (2 * wb + (rem & 1)) * PX_PATCH;
+  const int f0 = 2 * t, f1 = f0 + 1 < im.frames ? f0 + 1 : im.frames - 1;
+  const int lb = im.width * 3;
+  const int64_t fb = (int64_t)lb * im.height;
+  const int64_t first = f0 * fb + (int64_t)y0 * lb + x0 * 3;
+  line_bytes = lb;
+  frame_off = (int)((f1 - f0) * fb);
+  base = im.pixels + first;
+}
+// The 8 bytes at p (2-byte aligned when the frame buffer is 4-byte aligned; global memory takes unaligned vector loads),
+// as one load whose result is not touched until px_convert8, so that it can stay in flight.
+struct PxRaw {
+  u32x2 w;
+};
+__device__ __forceinline__ void px_fetch8(const uint8_t* p, PxRaw& r) {
+  typedef __attribute__((address_space(1))) const uint8_t* global_bytes;  // frames are in device memory: no generic-address load
+  __builtin_memcpy(&r.w, (global_bytes)(uintptr_t)p, 8);
+}
+// the normalisation constants as six scalars (kernel arguments indexed by a lane-varying channel would be fetched from
+// memory for every use)
+struct PxNorm {
+  float a0, a1, a2, c0, c1, c2;
+  __device__ __forceinline__ explicit PxNorm(const GemmParams& p) : a0(p.px_a[0]), a1(p.px_a[1]), a2(p.px_a[2]), c0(p.px_c[0]), c1(p.px_c[1]), c2(p.px_c[2]) {}
+};
+// 8 bytes -> bf16(byte * a + c), the first byte belonging to channel ch0.  tail: the load was moved 6 bytes back so that
+// it ends with the line (piece 5 holds bytes 40, 41 of the line and six padding columns): its last two bytes are the
+// piece's first two, the rest of the piece is padding.
+__device__ __forceinline__ bf16x8 px_convert8(const PxRaw& r, int ch0, bool tail, const PxNorm nm) {
+  const unsigned raw[2] = {tail ? r.w[1] >> 16 : r.w[0], tail ? 0u : r.w[1]};
+  // a, c of bytes 0, 1, 2 (mod 3) of the piece: the constants rotated by ch0
+  const bool r1 = ch0 == 1, r2 = ch0 == 2;
+  const float ar0 = r2 ? nm.a2 : (r1 ? nm.a1 : nm.a0), ar1 = r2 ? nm.a0 : (r1 ? nm.a2 : nm.a1), ar2 = r2 ? nm.a1 : (r1 ? nm.a0 : nm.a2);
+  const float cr0 = r2 ? nm.c2 : (r1 ? nm.c1 : nm.c0), cr1 = r2 ? nm.c0 : (r1 ? nm.c2 : nm.c1), cr2 = r2 ? nm.c1 : (r1 ? nm.c0 : nm.c2);
+  bf16x8 v;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float x = (float)((raw[e >> 2] >> (8 * (e & 3))) & 0xffu);
+    v[e] = (bf16_t)__builtin_fmaf(x, e % 3 == 0 ? ar0 : (e % 3 == 1 ? ar1 : ar2), e % 3 == 0 ? cr0 : (e % 3 == 1 ? cr1 : cr2));
+  }
+  return v;
+}
 // MFMA operand fetch from LDS for the 32-row sub-tile starting at `row`, contraction offset `k`.
 template <bool TR, int ROWS>
 __device__ __forceinline__ bf16x8 frag_bf16(const bf16_t* lds, int row, int k) {
@@ -851,6 +927,50 @@ struct DlOperand {
   }
 };
 
+// The loader of that operand for the DL layout: this operand cannot travel global -> LDS directly, so a K tile takes two calls, a step of the main loop apart:
+// request() loads this lane's 8 bytes of each of its CPT rows into registers, flush() converts them and writes the 16-byte
+// chunk where the direct load of a [row][k] operand would have put it (slot l of the wave's 1 KiB slice holds chunk
+// (l & 3) ^ ((row >> 2) & 3) of row 16 * slice + l / 4).  A K tile of 32 is 4 pieces, so pieces advance by 4 per tile.
+template <int NW>
+struct DlPixelOperand {
+  static constexpr int CPT = DL<NW>::CPT;
+  static_assert(PX_K % DL_BK == 0, "whole K tiles");
+  const uint8_t* base[CPT];
+  int line_bytes[CPT], frame_off[CPT];
+  int line, piece;  // of the next request
+  int ch0;          // channel of the first byte of the piece that the next flush converts
+  PxRaw raw[CPT];
+
+  __device__ __forceinline__ void init(const GemmParams& p, int64_t row0, int wv) {
+    const int l = threadIdx.x & 63;
+    line = 0;
+    piece = (l & 3) ^ ((l >> 4) & 3);  // (row >> 2) & 3 = (l >> 4) & 3: slices start at multiples of 16 rows
+    ch0 = (2 * piece) % 3;
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) px_locate(p, row0 + (wv * CPT + i) * 16 + (l >> 2), base[i], line_bytes[i], frame_off[i]);
+  }
+  __device__ __forceinline__ void request() {
+    const int second = line >= PX_PATCH ? 1 : 0, y = line - PX_PATCH * second;
+    const int in_line = piece == 5 ? 8 * 5 - 6 : 8 * piece;  // the last piece is read as the last 8 bytes of the line
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) px_fetch8(base[i] + ((second ? frame_off[i] : 0) + y * line_bytes[i] + in_line), raw[i]);
+    piece += 4;
+    if (piece >= 6) {
+      piece -= 6;
+      line += 1;
+    }
+  }
+  // lds_slice: this wave's CPT KiB of the operand's stage.  The write is complete before the wave's next barrier
+  // because the fragment reads that follow it in program order are (LDS operations of a wave complete in order).
+  __device__ __forceinline__ void flush(unsigned char* lds_slice, const PxNorm nm) {
+    const int l = threadIdx.x & 63;
+    const bool tail = piece == 3;  // the piece in registers is 4 pieces (mod 6) before the next request's
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) *reinterpret_cast<bf16x8*>(lds_slice + i * 1024 + l * 16) = px_convert8(raw[i], ch0, tail, nm);
+    ch0 = ch0 == 0 ? 2 : ch0 - 1;  // 32 bytes further: + 2 mod 3 (a wrap to the next line moves by 48 = 0 mod 3)
+  }
+};
+
 // MFMA operand fetch for the DL layout: sub-tile `a` (32 rows) of the wave, 16-wide contraction step ks, stage s.
 template <bool TR, int NSUB, bool MI16 = false>
 struct DlFrag {
@@ -932,8 +1052,10 @@ __device__ __forceinline__ void wait_tiles(int n) {
   else wait_vm<0>();
 }
 
-template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, int NW, bool MI16 = false>
+// PIX: the A operand is made from decoded frames (DlPixelOperand)
+template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, int NW, bool MI16 = false, bool PIX = false>
 __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmParams p) {
+  static_assert(!PIX || (!TA && !MI16 && !dl_prefetches(EPI, TA)), "frames as the A operand: [row][k] layout, 32x32x16 fragments, no early loads");
   using T = bf16_t;
   using D = DL<NW>;
   constexpr int BM = D::BM, BN = D::BN, WM = D::WM, WN = D::WN, TILE = D::TILE_BYTES, SLICE = D::CPT * 1024;
@@ -961,17 +1083,31 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
   constexpr bool PREFETCH = dl_prefetches(EPI, TA);
   constexpr int EARLY = PREFETCH ? (NSTAGE - 1 < 2 ? NSTAGE - 1 : 2) : NSTAGE - 1;  // K tiles requested by start_tile
   constexpr int STAGING_OFF = PREFETCH ? (NSTAGE + EARLY) * TILE : 0;
-  DlOperand<TA, false, NW, MI16> la;
+  typename std::conditional<PIX, DlPixelOperand<NW>, DlOperand<TA, false, NW, MI16>>::type la;
   DlOperand<TB, DUAL, NW, MI16> lb;
   int T_ = 0, k_tail = 0;  // of the tile whose operands are being loaded
+  [[maybe_unused]] int px_pending = -1;  // PIX: stage whose A bytes are in registers, requested by the previous issue()
+  [[maybe_unused]] const PxNorm px_norm(p);
+  const bool px_late = PIX && wv >= NW / 2;
   auto issue = [&](int t, int s) {  // K tile t into stage s (both wave-uniform)
-    if (t >= T_) return;
-    if (k_tail != 0 && t == T_ - 1) {
-      la.issue_tail(smem_raw + s * TILE + wv * SLICE, k_tail, wv);
-      lb.issue_tail(smem_raw + (NSTAGE + s) * TILE + wv * SLICE, k_tail, wv);
-    } else {
-      la.issue(lds0 + s * TILE);
+    if constexpr (PIX) {
+      // the A bytes requested one call ago are converted and written now (their K tile is read two barriers from here),
+      // then K tile t is requested: B straight into LDS, A into registers
+      if (px_pending >= 0) la.flush(smem_raw + px_pending * TILE + wv * SLICE, px_norm);
+      px_pending = -1;
+      if (t >= T_) return;
       lb.issue(lds0 + (NSTAGE + s) * TILE);
+      la.request();
+      px_pending = s;
+    } else {
+      if (t >= T_) return;
+      if (k_tail != 0 && t == T_ - 1) {
+        la.issue_tail(smem_raw + s * TILE + wv * SLICE, k_tail, wv);
+        lb.issue_tail(smem_raw + (NSTAGE + s) * TILE + wv * SLICE, k_tail, wv);
+      } else {
+        la.issue(lds0 + s * TILE);
+        lb.issue(lds0 + (NSTAGE + s) * TILE);
+      }
     }
   };
   constexpr int N_PER_BLOCK = DUAL ? BN / 2 : BN;
@@ -989,7 +1125,8 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
     const int64_t k_end = p.split_k > 1 ? (k_begin + p.k_chunk < p.K ? k_begin + p.k_chunk : p.K) : p.K;
     next_m0 = (int64_t)tm * BM;
     next_n0 = (int64_t)tn * N_PER_BLOCK;
-    la.init(static_cast<const T*>(p.A), nullptr, p.lda, next_m0, p.M, k_begin, wv);
+    if constexpr (PIX) la.init(p, next_m0, wv);
+    else la.init(static_cast<const T*>(p.A), nullptr, p.lda, next_m0, p.M, k_begin, wv);
     lb.init(static_cast<const T*>(p.B), static_cast<const T*>(p.B2), p.ldb, next_n0, p.N, k_begin, wv);
     const int klen = (int)(k_end - k_begin);
     T_ = (klen + DL_BK - 1) / DL_BK;
@@ -1033,7 +1170,10 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
       constexpr int AHEAD = NSTAGE - 2;
       wait_tiles<2 * D::CPT>(rem < 0 ? 0 : (rem < AHEAD ? rem : AHEAD));
       __builtin_amdgcn_s_barrier();  // every wave's share of that tile is in LDS; stage (s-1) has been consumed
-      issue(t + NSTAGE - 1, (s + NSTAGE - 1) % NSTAGE);
+      // PIX: the conversion of the A bytes is vector work of about the length of a K tile's MFMAs.  The two waves of a
+      // SIMD (w and w + NW/2) do it at opposite ends of the step, one before its MFMAs and one after, so that one
+      // wave's conversions run under the other's MFMAs.
+      if (!px_late) issue(t + NSTAGE - 1, (s + NSTAGE - 1) % NSTAGE);
 
       if constexpr (MI16) {
         // one 32-wide step per stage on v_mfma_f32_16x16x32_bf16: 2*MT x 2*NT blocks of 16x16
@@ -1080,6 +1220,12 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
         for (int b = 0; b < NT; ++b)
           acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][a], fb[1][b], acc[a][b], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (PIX) {
+        if (px_late) {
+          issue(t + NSTAGE - 1, (s + NSTAGE - 1) % NSTAGE);
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // no LDS read follows the write before the barrier
+        }
       }
     }
   }
@@ -1133,7 +1279,7 @@ int launch(const GemmParams& p, hipStream_t stream) {
   return MVIT_OK;
 }
 
-template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, int NW, bool MI16 = false>
+template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, int NW, bool MI16 = false, bool PIX = false>
 int launch_dl(const GemmParams& p, hipStream_t stream) {
   using D = DL<NW>;
   constexpr size_t operands = 2 * (size_t)NSTAGE * D::TILE_BYTES;
@@ -1142,7 +1288,7 @@ int launch_dl(const GemmParams& p, hipStream_t stream) {
   constexpr size_t staging_end = dl_prefetches(EPI, TA) ? (NSTAGE + (NSTAGE - 1 < 2 ? NSTAGE - 1 : 2)) * D::TILE_BYTES + staging : staging;
   constexpr size_t lds = staging_end > operands ? staging_end : operands;
   static_assert(lds <= 160 * 1024, "operand stages plus the epilogue staging area exceed the LDS of a CU");
-  auto kern = gemm_dl_kernel<TO, TA, TB, EPI, NSTAGE, NW, MI16>;
+  auto kern = gemm_dl_kernel<TO, TA, TB, EPI, NSTAGE, NW, MI16, PIX>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -1222,7 +1368,87 @@ inline bool vec16(const void* ptr, int64_t ld, size_t esize) {
   return ptr == nullptr || (mvit_aligned16(ptr) && (ld * (int64_t)esize) % 16 == 0);
 }
 
+// packed[n][line * 48 + b] = w[n][channel * 392 + frame * 196 + y * 14 + x] for b = x * 3 + channel < 42, else 0
+// (line = frame * 14 + y): the patch-embedding weight in the contraction order of DlPixelOperand
+template <typename T>
+__global__ __launch_bounds__(256) void pack_patch_weight_kernel(const T* __restrict__ w, int64_t ldw, int64_t n_out, bf16_t* __restrict__ packed) {
+  const int64_t total = n_out * PX_K;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t n = i / PX_K;
+    const int k = (int)(i % PX_K), ln = k / PX_LINE, b = k % PX_LINE;
+    float v = 0.f;
+    if (b < PX_PATCH * 3) {
+      const int x = b / 3, ch = b % 3, fr = ln / PX_PATCH, y = ln % PX_PATCH;
+      v = to_f32(w[n * ldw + ch * (2 * PX_PATCH * PX_PATCH) + fr * (PX_PATCH * PX_PATCH) + y * PX_PATCH + x]);
+    }
+    packed[i] = from_f32<bf16_t>(v);
+  }
+}
+
+// float -> bf16 bits, round to nearest even (finite inputs)
+inline uint16_t host_bf16_bits(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
 }  // namespace
+
+extern "C" int mvit_patch_embed_pack_weight(const void* w, int dtype, int64_t ldw, int64_t n_out, void* packed, mvit_stream_t stream) {
+  MVIT_REQUIRE(w && packed, "patch_embed_pack_weight: null pointer");
+  MVIT_REQUIRE(dtype == MVIT_BF16 || dtype == MVIT_F32, "patch_embed_pack_weight: dtype %d", dtype);
+  MVIT_REQUIRE(n_out > 0 && ldw >= MVIT_PIXEL_ROW, "patch_embed_pack_weight: n_out=%lld ldw=%lld", (long long)n_out, (long long)ldw);
+  MVIT_REQUIRE(mvit_aligned16(packed), "patch_embed_pack_weight: packed must be 16-byte aligned");
+  const int64_t total = n_out * PX_K;
+  const int grid = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (dtype == MVIT_BF16) hipLaunchKernelGGL((pack_patch_weight_kernel<bf16_t>), grid, 256, 0, s, static_cast<const bf16_t*>(w), ldw, n_out, static_cast<bf16_t*>(packed));
+  else hipLaunchKernelGGL((pack_patch_weight_kernel<float>), grid, 256, 0, s, static_cast<const float*>(w), ldw, n_out, static_cast<bf16_t*>(packed));
+  MVIT_CHECK_LAUNCH("patch_embed_pack_weight");
+  return MVIT_OK;
+}
+
+extern "C" int mvit_patch_embed_frames(const mvit_image* images, int n_images, int64_t total_rows, const void* packed_w, int64_t n_out,
+                                       void* out, int64_t ldo, int out_dtype, double rescale, float mean_r, float mean_g, float mean_b,
+                                       float std_r, float std_g, float std_b, mvit_stream_t stream) {
+  MVIT_REQUIRE(images && packed_w && out, "patch_embed_frames: null pointer");
+  MVIT_REQUIRE(n_images > 0 && total_rows >= 0 && n_out > 0 && ldo >= n_out, "patch_embed_frames: n_images=%d total_rows=%lld n_out=%lld ldo=%lld",
+               n_images, (long long)total_rows, (long long)n_out, (long long)ldo);
+  MVIT_REQUIRE(out_dtype == MVIT_BF16 || out_dtype == MVIT_F32, "patch_embed_frames: out_dtype %d", out_dtype);
+  MVIT_REQUIRE(mvit_aligned16(packed_w), "patch_embed_frames: packed_w must be 16-byte aligned");
+  if (total_rows == 0) return MVIT_OK;
+  GemmParams p;
+  memset(&p, 0, sizeof(p));
+  // the kernel computes byte * a + c in one fused multiply-add; that is only taken when, rounded to bf16, it gives
+  // the table of mvit_patchify ((float)((double)byte * rescale) - mean) / std for all 256 bytes of every channel
+  const float mean[3] = {mean_r, mean_g, mean_b}, stdv[3] = {std_r, std_g, std_b};
+  for (int c = 0; c < 3; ++c) {
+    MVIT_REQUIRE(stdv[c] != 0.f, "patch_embed_frames: std[%d] = 0", c);
+    p.px_a[c] = (float)(rescale / (double)stdv[c]);
+    p.px_c[c] = (float)(-(double)mean[c] / (double)stdv[c]);
+    for (int b = 0; b < 256; ++b) {
+      const float x = (float)((double)b * rescale);
+      volatile float diff = x - mean[c];
+      const float table = diff / stdv[c];
+      const float affine = fmaf((float)b, p.px_a[c], p.px_c[c]);
+      if (host_bf16_bits(table) != host_bf16_bits(affine))
+        return mvit_set_error(MVIT_ERR_UNSUPPORTED, "patch_embed_frames: byte %d of channel %d: a * x + c does not round to the bf16 value of "
+                              "(x * rescale - mean) / std for these constants; use mvit_patchify + mvit_gemm", b, c);
+    }
+  }
+  p.M = total_rows; p.N = n_out; p.K = PX_K;
+  p.B = packed_w; p.ldb = PX_K; p.C = out; p.ldc = ldo;
+  p.px_images = images; p.px_n_images = n_images;
+  p.vec_ok = vec16(out, ldo, out_dtype == MVIT_BF16 ? 2 : 4);
+  const int64_t tm = (total_rows + 255) / 256, tn = (n_out + 255) / 256;
+  MVIT_REQUIRE(tm * tn < (1ll << 30), "patch_embed_frames: too many tiles");
+  p.tiles_m = (int)tm; p.tiles_n = (int)tn;
+  p.panel_w = tn <= 6 ? (int)tn : 4;
+  p.split_k = 1; p.k_chunk = PX_K;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (out_dtype == MVIT_BF16) return launch_dl<bf16_t, false, false, MVIT_EPI_NONE, 4, 8, false, true>(p, s);
+  return launch_dl<float, false, false, MVIT_EPI_NONE, 4, 8, false, true>(p, s);
+}
 
 extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
   MVIT_REQUIRE(a, "gemm: null args");

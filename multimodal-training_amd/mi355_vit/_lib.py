@@ -79,6 +79,8 @@ PROTOTYPES = {
     "mvit_grad_sumsq_static": [_vp, _i32, _i64, _vp, _i32, _vp],
     "mvit_patchify": [_vp, _i32, _i64, _vp, C.c_double] + [_f32] * 6 + [_i32, _vp],
     "mvit_resample_u8": [_vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _i32, _vp],
+    "mvit_patch_embed_pack_weight": [_vp, _i32, _i64, _i64, _vp, _vp],
+    "mvit_patch_embed_frames": [_vp, _i32, _i64, _vp, _i64, _vp, _i64, _i32, C.c_double] + [_f32] * 6 + [_vp],
     "mvit_attn_bwd": [_vp] * 12 + [_i32, _i32, _i64, _i32, _i32] + [_i64] * 8 + [_f32, _i32, _vp],
 }
 EXPORTS = sorted(list(PROTOTYPES) + ["mvit_version", "mvit_last_error"])
@@ -108,7 +110,11 @@ def load() -> C.CDLL:
     return _lib
 
 
+class Unsupported(RuntimeError):
+    """MVIT_ERR_UNSUPPORTED: the library has no kernel for this case (arguments were well-formed)."""
+
+
 def check(rc: int, what: str) -> None:
     if rc != 0:
         msg = load().mvit_last_error().decode("utf-8", "replace")
-        raise RuntimeError(f"{what} failed (code {rc}): {msg}")
+        raise (Unsupported if rc == -3 else RuntimeError)(f"{what} failed (code {rc}): {msg}")

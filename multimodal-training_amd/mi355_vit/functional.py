@@ -280,6 +280,32 @@ class PatchEmbedFn(torch.autograd.Function):
         return None, gw.view(ctx.wshape), None
 
 
+class PatchEmbedFramesFn(torch.autograd.Function):
+    """The patch embedding straight from decoded uint8 frames (bf16 compute): the forward makes the rows of
+    ``pixel_values`` inside the GEMM and never writes them; the weight gradient needs them as a matrix, so the backward
+    writes them once (``patchify``) just before its GEMM and drops them again."""
+
+    @staticmethod
+    def forward(ctx, weight, out_dtype, *frames):
+        from . import pixels
+
+        out, _ = pixels.patch_embed_frames(frames, pixels.pack_patch_embed_weight(weight), dtype=out_dtype)
+        ctx.frames, ctx.wshape, ctx.wdtype = frames, weight.shape, weight.dtype
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        from . import pixels
+
+        px, _ = pixels.patchify(ctx.frames, dtype=torch.bfloat16)
+        dy = dout.contiguous()
+        if dy.dtype != torch.bfloat16:
+            dy = ops.cast2d(dy, torch.empty(dy.shape, dtype=torch.bfloat16, device=dy.device))
+        gw = torch.empty(dy.shape[1], px.shape[1], dtype=ctx.wdtype, device=px.device)
+        ops.gemm(dy, px, gw, trans_a=True, trans_b=True, split_k=ops.wgrad_split_k(gw.shape[0], gw.shape[1], px.shape[0]))
+        return (gw.view(ctx.wshape), None) + (None,) * len(ctx.frames)
+
+
 class PermuteRowsFn(torch.autograd.Function):
     """out.view(n, unit*cols)[i] = x.view(n, unit*cols)[index[i]]; `inverse` is the inverse permutation."""
 

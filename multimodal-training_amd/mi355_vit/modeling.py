@@ -21,6 +21,7 @@ from .functional import (
     AttnGeometry,
     MergerFn,
     PatchEmbedFn,
+    PatchEmbedFramesFn,
     PermuteRowsFn,
     VisionBlockFn,
     pack_block_weights,
@@ -61,6 +62,24 @@ class Qwen2_5_VisionPatchEmbed(nn.Module):
 
     def forward(self, hidden_states: torch.Tensor, compute_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         return PatchEmbedFn.apply(hidden_states, self.proj.weight, compute_dtype or self.proj.weight.dtype)
+
+    fuse_frames = True  # bf16: make the rows of pixel_values inside the GEMM instead of writing them first
+
+    def forward_frames(self, frames, compute_dtype: Optional[torch.dtype] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Decoded, resized uint8 frame stacks (``[frames, H, W, 3]`` per image or video, on the GPU) -> (patch
+        embeddings, ``image_grid_thw``): the image processor's rescale / normalise / patchify and this module's
+        projection in one step."""
+        from . import _lib, pixels
+
+        T = compute_dtype or self.proj.weight.dtype
+        frames = list(frames)
+        if self.fuse_frames and T == torch.bfloat16 and pixels.frames_fit_fused_patch_embed(frames):
+            try:
+                return PatchEmbedFramesFn.apply(self.proj.weight, T, *frames), pixels.grid_thw_of(frames)
+            except _lib.Unsupported:  # normalisation constants that do not fold into one multiply-add per byte
+                pass
+        rows, grid = pixels.patchify(frames, dtype=T)
+        return self.forward(rows, T), grid
 
 
 class Qwen2_5_VisionRotaryEmbedding(nn.Module):
@@ -274,9 +293,12 @@ class Qwen2_5_VisionTransformerPretrainedModel(nn.Module):
         return self.dtype
 
     # ---- forward ---------------------------------------------------------------------------------
-    def forward(self, hidden_states: torch.Tensor, grid_thw: torch.Tensor, **kwargs) -> torch.Tensor:
+    def forward(self, hidden_states: Optional[torch.Tensor] = None, grid_thw: Optional[torch.Tensor] = None, *, frames=None,
+                **kwargs) -> torch.Tensor:
         """hidden_states: pixels view-able to [-1, in_channels*temporal_patch*patch*patch]; grid_thw [N,3] int64.
-        Returns [S / merge^2, out_hidden_size] in the original (un-windowed) token order."""
+        Returns [S / merge^2, out_hidden_size] in the original (un-windowed) token order.
+        ``frames`` (instead of ``hidden_states``; ``grid_thw`` then follows from their shapes): decoded, resized uint8
+        frame stacks ``[frames, H, W, 3]`` on the GPU, one per image or video."""
         if self.sequence_parallel:
             raise NotImplementedError(
                 "sequence_parallel=True needs inter-GPU collectives, which this single-GPU build does not have; "
@@ -288,10 +310,20 @@ class Qwen2_5_VisionTransformerPretrainedModel(nn.Module):
         T = self._compute_dtype()
         if T not in (torch.float32, torch.bfloat16):
             raise TypeError(f"compute dtype {T} is not supported (float32 or bfloat16)")
+        if (hidden_states is None) == (frames is None):
+            raise ValueError("pass either hidden_states (with grid_thw) or frames")
+        if frames is not None:
+            x, grid_of_frames = self.patch_embed.forward_frames(frames, T)
+            if grid_thw is not None and grid_thw.detach().to("cpu", torch.int64).reshape(-1, 3).tolist() != grid_of_frames.tolist():
+                raise ValueError(f"grid_thw {grid_thw.tolist()} does not describe the frames ({grid_of_frames.tolist()})")
+            grid_thw = grid_of_frames
+        elif grid_thw is None:
+            raise ValueError("hidden_states needs grid_thw")
         plan = self._plan(grid_thw, device)
         unit = self.spatial_merge_unit
 
-        x = self.patch_embed(hidden_states.to(device), T)
+        if frames is None:
+            x = self.patch_embed(hidden_states.to(device), T)
         if x.shape[0] != plan.seq_len:
             raise ValueError(f"hidden_states holds {x.shape[0]} patches but grid_thw describes {plan.seq_len}")
         x = PermuteRowsFn.apply(x, plan.window_index, plan.reverse_index, unit)

@@ -53,17 +53,12 @@ def grid_thw_of(frames: Sequence[torch.Tensor]) -> torch.Tensor:
     return torch.tensor(rows, dtype=torch.int64).reshape(-1, 3)
 
 
-def patchify(frames: Sequence[torch.Tensor], dtype: torch.dtype = torch.float32,
-             image_mean: Sequence[float] = OPENAI_CLIP_MEAN, image_std: Sequence[float] = OPENAI_CLIP_STD,
-             rescale_factor: float = 1.0 / 255.0, out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Frames of a batch of images / videos -> (``pixel_values`` [rows, 1176] on the GPU, ``image_grid_thw`` [n, 3]).
-
-    ``frames``: one contiguous uint8 GPU tensor ``[frames, height, width, 3]`` per image (one frame) or video.
-    ``dtype``: float32 (what the processor returns) or bfloat16 (what the tower casts it to).
-    """
+def _image_table(frames: Sequence[torch.Tensor], what: str):
+    """Checks the frame stacks and builds the device table of ``mvit_image`` entries (32 bytes per image, one
+    synchronous copy).  Returns (frames as a list, image_grid_thw, device table, total rows)."""
     frames = list(frames)
     if not frames:
-        raise ValueError("patchify: no images")
+        raise ValueError(f"{what}: no images")
     grid = grid_thw_of(frames)
     device = frames[0].device
     for i, f in enumerate(frames):
@@ -71,12 +66,6 @@ def patchify(frames: Sequence[torch.Tensor], dtype: torch.dtype = torch.float32,
             raise RuntimeError(f"image {i} on {f.device}: frames must be on one GPU (there is no CPU path)")
         if not f.is_contiguous():
             raise RuntimeError(f"image {i}: frames must be contiguous")
-    if dtype == torch.float32:
-        code = _lib.F32
-    elif dtype == torch.bfloat16:
-        code = _lib.BF16
-    else:
-        raise TypeError(f"unsupported dtype {dtype} (float32 and bfloat16 only)")
     counts = (grid[:, 0] * grid[:, 1] * grid[:, 2]).numpy()
     n = len(frames)
     table = np.zeros(n + 1, dtype=_TABLE_DTYPE)
@@ -86,11 +75,29 @@ def patchify(frames: Sequence[torch.Tensor], dtype: torch.dtype = torch.float32,
     table["width"][:n] = [f.shape[2] for f in frames]
     table["first_row"][1:] = np.cumsum(counts)
     total = int(table["first_row"][n])
+    return frames, grid, torch.from_numpy(table.view(np.uint8)).to(device), total
+
+
+def patchify(frames: Sequence[torch.Tensor], dtype: torch.dtype = torch.float32,
+             image_mean: Sequence[float] = OPENAI_CLIP_MEAN, image_std: Sequence[float] = OPENAI_CLIP_STD,
+             rescale_factor: float = 1.0 / 255.0, out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Frames of a batch of images / videos -> (``pixel_values`` [rows, 1176] on the GPU, ``image_grid_thw`` [n, 3]).
+
+    ``frames``: one contiguous uint8 GPU tensor ``[frames, height, width, 3]`` per image (one frame) or video.
+    ``dtype``: float32 (what the processor returns) or bfloat16 (what the tower casts it to).
+    """
+    if dtype == torch.float32:
+        code = _lib.F32
+    elif dtype == torch.bfloat16:
+        code = _lib.BF16
+    else:
+        raise TypeError(f"unsupported dtype {dtype} (float32 and bfloat16 only)")
+    frames, grid, dev_table, total = _image_table(frames, "patchify")
+    n, device = len(frames), frames[0].device
     if out is None:
         out = torch.empty((total, _lib.PIXEL_ROW), dtype=dtype, device=device)
     elif out.shape != (total, _lib.PIXEL_ROW) or out.dtype != dtype or out.device != device or not out.is_contiguous():
         raise RuntimeError(f"patchify: out must be a contiguous {dtype} [{total}, {_lib.PIXEL_ROW}] tensor on {device}")
-    dev_table = torch.from_numpy(table.view(np.uint8)).to(device)  # 32 bytes per image, synchronous copy
     mean = [float(np.float32(m)) for m in image_mean]
     std = [float(np.float32(s)) for s in image_std]
     lib = _lib.load()
@@ -98,6 +105,59 @@ def patchify(frames: Sequence[torch.Tensor], dtype: torch.dtype = torch.float32,
         stream = torch.cuda.current_stream(device).cuda_stream
         rc = lib.mvit_patchify(dev_table.data_ptr(), n, total, out.data_ptr(), float(rescale_factor), *mean, *std, code, stream)
     _lib.check(rc, "mvit_patchify")
+    return out, grid
+
+
+PACKED_PATCH_K = 1344  # 28 pixel lines of a patch (frame of the pair, y), each 14 x 3 bytes padded to 48
+
+
+def frames_fit_fused_patch_embed(frames: Sequence[torch.Tensor]) -> bool:
+    """Whether ``patch_embed_frames`` can read these frame stacks: 4-byte aligned buffers below 2 GiB each."""
+    return all(f.data_ptr() % 4 == 0 and f.numel() < 2**31 for f in frames)
+
+
+def pack_patch_embed_weight(weight: torch.Tensor) -> torch.Tensor:
+    """The patch-embedding weight ([embed_dim, 1176] or the Conv3d's [embed_dim, 3, 2, 14, 14], float32 or bfloat16)
+    in the contraction order of ``patch_embed_frames``: bfloat16 ``[embed_dim, 1344]``."""
+    w = weight.detach().reshape(weight.shape[0], -1)
+    if w.shape[1] != _lib.PIXEL_ROW or w.dtype not in (torch.float32, torch.bfloat16) or not w.is_cuda:
+        raise ValueError(f"pack_patch_embed_weight: expected a float32 / bfloat16 GPU weight with {_lib.PIXEL_ROW} inputs, got {w.dtype} {tuple(w.shape)} on {w.device}")
+    if w.stride(1) != 1:
+        w = w.contiguous()
+    packed = torch.empty((w.shape[0], PACKED_PATCH_K), dtype=torch.bfloat16, device=w.device)
+    lib = _lib.load()
+    with torch.cuda.device(w.device):
+        rc = lib.mvit_patch_embed_pack_weight(w.data_ptr(), _lib.BF16 if w.dtype == torch.bfloat16 else _lib.F32, w.stride(0),
+                                              w.shape[0], packed.data_ptr(), torch.cuda.current_stream(w.device).cuda_stream)
+    _lib.check(rc, "mvit_patch_embed_pack_weight")
+    return packed
+
+
+def patch_embed_frames(frames: Sequence[torch.Tensor], packed_weight: torch.Tensor, dtype: torch.dtype = torch.bfloat16,
+                       image_mean: Sequence[float] = OPENAI_CLIP_MEAN, image_std: Sequence[float] = OPENAI_CLIP_STD,
+                       rescale_factor: float = 1.0 / 255.0) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Frames -> (patch embeddings ``[rows, embed_dim]``, ``image_grid_thw``): ``patchify(frames, bfloat16)`` times the
+    weight, in one kernel that makes the rows on the fly and never writes them.  ``packed_weight`` comes from
+    ``pack_patch_embed_weight``.  Raises ``_lib.Unsupported`` when the normalisation constants cannot be folded into
+    one multiply-add per byte without changing a bfloat16 value (the caller then uses ``patchify`` and a GEMM)."""
+    if dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError(f"unsupported dtype {dtype} (float32 and bfloat16 only)")
+    frames, grid, dev_table, total = _image_table(frames, "patch_embed_frames")
+    device = frames[0].device
+    if not frames_fit_fused_patch_embed(frames):
+        raise RuntimeError("patch_embed_frames: frame buffers must be 4-byte aligned and smaller than 2 GiB")
+    if (packed_weight.dim() != 2 or packed_weight.shape[1] != PACKED_PATCH_K or packed_weight.dtype != torch.bfloat16
+            or packed_weight.device != device or not packed_weight.is_contiguous()):
+        raise ValueError("patch_embed_frames: packed_weight must be the contiguous bfloat16 [embed_dim, 1344] result of pack_patch_embed_weight on the frames' GPU")
+    out = torch.empty((total, packed_weight.shape[0]), dtype=dtype, device=device)
+    mean = [float(np.float32(m)) for m in image_mean]
+    std = [float(np.float32(s)) for s in image_std]
+    lib = _lib.load()
+    with torch.cuda.device(device):
+        rc = lib.mvit_patch_embed_frames(dev_table.data_ptr(), len(frames), total, packed_weight.data_ptr(), packed_weight.shape[0],
+                                         out.data_ptr(), out.stride(0), _lib.BF16 if dtype == torch.bfloat16 else _lib.F32,
+                                         float(rescale_factor), *mean, *std, torch.cuda.current_stream(device).cuda_stream)
+    _lib.check(rc, "mvit_patch_embed_frames")
     return out, grid
 
 

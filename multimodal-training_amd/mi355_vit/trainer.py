@@ -354,15 +354,14 @@ class BaseVisionTrainer(Trainer):
                 frames.append(resize_frames(f, th, tw))
             batch["frames"] = frames
         if batch.get("pixel_values") is None and batch.get("frames") is not None:
-            # resized uint8 frames ([frames, H, W, 3] per image or video) instead of the processor's float rows:
-            # a fifth of the upload, and rescale / normalise / patchify run on the GPU in the model's dtype
-            from .pixels import patchify
+            # resized uint8 frames ([frames, H, W, 3] per image or video) instead of the processor's float rows: a fifth
+            # of the upload; rescale / normalise / patchify run on the GPU, inside the patch-embedding GEMM
+            from .pixels import grid_thw_of
 
-            frames = [f.to(device, non_blocking=True).contiguous() for f in batch["frames"]]
-            param_dtype = next(self.model.parameters()).dtype
-            batch["pixel_values"], batch["image_grid_thw"] = patchify(
-                frames, dtype=param_dtype if param_dtype in (torch.float32, torch.bfloat16) else torch.float32)
-        batch["pixel_values"] = batch["pixel_values"].to(device, non_blocking=True)
+            batch["frames"] = [f.to(device, non_blocking=True).contiguous() for f in batch["frames"]]
+            batch["image_grid_thw"] = grid_thw_of(batch["frames"])
+        else:
+            batch["pixel_values"] = batch["pixel_values"].to(device, non_blocking=True)
         batch["image_grid_thw"] = batch["image_grid_thw"].to(device, non_blocking=True)
         vision_outputs = self._model_forward(batch)
         forward_time_ms = 0.0
@@ -438,8 +437,10 @@ class BaseVisionTrainer(Trainer):
 
 class QwenVisionTrainer(BaseVisionTrainer):
     def _model_forward(self, batch):
-        pixel_values, grid = batch["pixel_values"], batch["image_grid_thw"]
+        pixel_values, grid = batch.get("pixel_values"), batch["image_grid_thw"]
         with self._get_autocast_context():
+            if pixel_values is None:  # uint8 frames: the model makes the patch rows itself
+                return self.model(frames=batch["frames"], grid_thw=grid).unsqueeze(0)
             if pixel_values.dim() == 5:  # [B, C, T, H, W] collated images that share one grid
                 B = pixel_values.shape[0]
                 if grid.dim() == 1:

@@ -136,7 +136,21 @@ def test_trainer_takes_frames_batches():
         tr.set_data_iterator([batch])
         tr.initialize_trainer()
         outs.append(tr.forward_step(0)["vision_embeddings"].detach().clone())
-    assert torch.equal(outs[0], outs[1])
+    # the frames path contracts the patch embedding in another order (along memory): same values up to bf16 rounding
+    err = (outs[0].float() - outs[1].float()).abs().max() / outs[1].float().abs().max()
+    assert err < 1e-2, err
+    # with the fusion switched off the two paths run the same kernels on the same bits
+    from mi355_vit.modeling import Qwen2_5_VisionPatchEmbed
+
+    Qwen2_5_VisionPatchEmbed.fuse_frames = False
+    try:
+        tr = VisionTrainer(cfg, rank=0)
+        tr.build_model()
+        tr.set_data_iterator([{"frames": [torch.from_numpy(im) for im in images], "sample_index": torch.tensor([0])}])
+        tr.initialize_trainer()
+        assert torch.equal(tr.forward_step(0)["vision_embeddings"], outs[1])
+    finally:
+        Qwen2_5_VisionPatchEmbed.fuse_frames = True
 
 
 def test_patchify_rejects_what_it_cannot_do():
@@ -155,6 +169,166 @@ def test_patchify_rejects_what_it_cannot_do():
         patchify([])
     with pytest.raises(RuntimeError, match="contiguous"):
         patchify([torch.zeros(1, 28, 56, 3, dtype=torch.uint8, device=DEV)[:, :, ::2]])
+
+
+# ------------------------------------------------------------------------------- patch embedding from frames
+
+
+def _bf16_rows_f64(images):
+    """pixel_values of the oracle, rounded to bfloat16 (what the tower multiplies), as float64."""
+    return torch.from_numpy(po.patchify_batch(images)[0]).to(torch.bfloat16).to(torch.float64)
+
+
+def test_pack_patch_embed_weight_is_the_documented_permutation():
+    from mi355_vit.pixels import pack_patch_embed_weight
+
+    _announce("pack patch-embed weight")
+    torch.manual_seed(0)
+    for dtype in (torch.bfloat16, torch.float32):
+        w = torch.randn(40, 3, 2, 14, 14, device=DEV).to(dtype)
+        got = pack_patch_embed_weight(w).cpu()
+        ref = torch.zeros(40, 28, 48, dtype=torch.bfloat16)
+        # [n, channel, frame, y, x] -> [n, frame, y, x, channel] -> lines of 42 values
+        ref[:, :, :42] = w.cpu().to(torch.bfloat16).permute(0, 2, 3, 4, 1).reshape(40, 28, 42)
+        assert got.shape == (40, 1344) and torch.equal(got, ref.reshape(40, 1344))
+
+
+@pytest.mark.parametrize("n_out,out_dtype", [(256, torch.float32), (200, torch.float32), (1280, torch.bfloat16)])
+def test_patch_embed_frames_equals_bf16_rows_times_weight(n_out, out_dtype):
+    """Ragged images and videos (odd frame counts, 616 rows = two full row tiles and a partial one): the fused kernel
+    equals oracle rows rounded to bf16 times the weight, evaluated in float64, to fp32-accumulation accuracy; one
+    operand element that differed by a bf16 ulp would show as ~1e-4 of the output scale."""
+    from mi355_vit.pixels import pack_patch_embed_weight, patch_embed_frames
+
+    _announce(f"patch_embed_frames ragged n_out={n_out} {out_dtype}")
+    images = _batch(11, RAGGED)
+    torch.manual_seed(1)
+    w = (torch.randn(n_out, 1176) * 0.05).to(torch.bfloat16)
+    got, grid = patch_embed_frames([torch.from_numpy(im).to(DEV) for im in images], pack_patch_embed_weight(w.to(DEV)), dtype=out_dtype)
+    torch.cuda.synchronize()
+    ref = _bf16_rows_f64(images) @ w.to(torch.float64).T
+    assert grid.tolist() == po.patchify_batch(images)[1].tolist() and tuple(got.shape) == tuple(ref.shape)
+    if out_dtype == torch.float32:
+        err = (got.cpu().double() - ref).abs().max() / ref.abs().max()
+        assert err < 2e-5, err
+    else:
+        assert got.dtype == torch.bfloat16
+        # at most one bf16 ulp from the rounded exact result (fp32 accumulation can tip a value that lies at a rounding boundary)
+        r = ref.to(torch.bfloat16).float()
+        ulp = torch.maximum(r.abs(), torch.tensor(1e-3)) * 2.0 ** -7
+        assert ((got.cpu().float() - r).abs() <= ulp).all()
+        assert (got.cpu().float() != r).float().mean() < 0.02
+
+
+def test_patch_embed_frames_full_benchmark_batch_against_the_two_kernel_path():
+    """cfg2's 8 ragged images (25,524 rows) at the tower's width: fused kernel against patchify + GEMM on the GPU and,
+    for sampled rows, against float64."""
+    from mi355_vit import ops
+    from mi355_vit.pixels import pack_patch_embed_weight, patch_embed_frames, patchify
+
+    _announce("patch_embed_frames cfg2 batch")
+    grids = [[1, 76, 60], [1, 86, 54], [1, 82, 34], [1, 42, 78], [1, 54, 32], [1, 72, 56], [1, 40, 42], [1, 64, 44]]
+    images = _batch(4, [(1, 14 * h, 14 * w) for _, h, w in grids])
+    frames = [torch.from_numpy(im).to(DEV) for im in images]
+    torch.manual_seed(2)
+    w = (torch.randn(1280, 1176, device=DEV) * 0.03).to(torch.bfloat16)
+    got, grid = patch_embed_frames(frames, pack_patch_embed_weight(w), dtype=torch.float32)
+    rows, _ = patchify(frames, dtype=torch.bfloat16)
+    two = torch.empty(rows.shape[0], 1280, dtype=torch.float32, device=DEV)
+    ops.gemm(rows, w, two)
+    torch.cuda.synchronize()
+    assert grid.tolist() == grids and got.shape == (25524, 1280)
+    scale = two.abs().max()
+    assert (got - two).abs().max() / scale < 2e-5
+    pick = torch.tensor([0, 1, 255, 256, 4559, 4560, 12000, 25523])
+    ref = rows[pick.to(DEV)].cpu().double() @ w.cpu().double().T
+    assert (got[pick.to(DEV)].cpu().double() - ref).abs().max() / ref.abs().max() < 2e-5
+
+
+def _affine_fold_is_exact(mean, std, scale):
+    """Whether byte * a + c (one fused multiply-add, float32) rounds to the same bfloat16 as the processor's
+    (float32(byte * scale) - mean) / std for every byte and channel: the library's own acceptance test, in numpy."""
+    def bf16_bits(x):
+        u = np.asarray(x, np.float32).view(np.uint32).astype(np.uint64)
+        return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint32)
+
+    b = np.arange(256)
+    for m, s in zip(mean, std):
+        m, s = np.float32(m), np.float32(s)
+        table = (((b.astype(np.float64) * scale).astype(np.float32) - m) / s).astype(np.float32)
+        a = np.float32(np.float64(scale) / np.float64(s))
+        c = np.float32(-np.float64(m) / np.float64(s))
+        affine = (b.astype(np.float64) * np.float64(a) + np.float64(c)).astype(np.float32)  # exact product and sum, one rounding
+        if not np.array_equal(bf16_bits(table), bf16_bits(affine)):
+            return False
+    return True
+
+
+def test_patch_embed_frames_refuses_constants_it_cannot_fold_and_the_module_falls_back():
+    from mi355_vit import _lib
+    from mi355_vit.pixels import OPENAI_CLIP_MEAN, OPENAI_CLIP_STD, pack_patch_embed_weight, patch_embed_frames
+
+    _announce("patch_embed_frames constants check")
+    assert _affine_fold_is_exact(OPENAI_CLIP_MEAN, OPENAI_CLIP_STD, 1.0 / 255.0)
+    rng = np.random.default_rng(5)
+    bad = None
+    for _ in range(2000):
+        mean, std = rng.uniform(0.2, 0.7, 3), rng.uniform(0.15, 0.4, 3)
+        if not _affine_fold_is_exact(mean, std, 1.0 / 255.0):
+            bad = (tuple(float(np.float32(x)) for x in mean), tuple(float(np.float32(x)) for x in std))
+            break
+    assert bad is not None
+    frames = [torch.from_numpy(im).to(DEV) for im in _batch(8, [(1, 28, 56)])]
+    pw = pack_patch_embed_weight(torch.randn(64, 1176, device=DEV).to(torch.bfloat16))
+    with pytest.raises(_lib.Unsupported, match="does not round"):
+        patch_embed_frames(frames, pw, image_mean=bad[0], image_std=bad[1])
+    with pytest.raises(RuntimeError, match="4-byte aligned"):
+        buf = torch.zeros(28 * 56 * 3 + 1, dtype=torch.uint8, device=DEV)
+        patch_embed_frames([buf[1:].view(1, 28, 56, 3)], pw)
+    with pytest.raises(ValueError, match="packed_weight"):
+        patch_embed_frames(frames, pw[:, :1176].contiguous())
+
+
+def test_tower_takes_frames_and_trains_the_patch_embedding():
+    """model(frames=...) equals model(pixel_values from patchify) up to bf16 rounding, and every gradient, the patch
+    embedding's included, matches; frames at an odd address take the two-kernel path and give the same bits as it."""
+    from mi355_vit.config import Qwen2_5_VLVisionConfig
+    from mi355_vit.modeling import Qwen2_5_VisionTransformerPretrainedModel
+    from mi355_vit.pixels import patchify
+
+    _announce("tower from frames")
+    images = _batch(9, [(1, 56, 84), (3, 56, 56), (1, 28, 28)])
+    frames = [torch.from_numpy(im).to(DEV) for im in images]
+    cfg = Qwen2_5_VLVisionConfig(depth=2, hidden_size=256, intermediate_size=300, num_heads=8, out_hidden_size=256,
+                                 window_size=56, fullatt_block_indexes=[1])
+    torch.manual_seed(0)
+    tower = Qwen2_5_VisionTransformerPretrainedModel(cfg).to(torch.bfloat16).to(DEV).train()
+    pv, grid = patchify(frames, dtype=torch.bfloat16)
+    gout = torch.randn(pv.shape[0] // 4, 256, device=DEV).to(torch.bfloat16)
+
+    def run(**kw):
+        tower.zero_grad(set_to_none=True)
+        out = tower(**kw)
+        out.backward(gout)
+        return out.detach().float(), {n: p.grad.detach().float().clone() for n, p in tower.named_parameters()}
+
+    out_f, g_f = run(frames=frames)
+    out_r, g_r = run(hidden_states=pv, grid_thw=grid)
+    assert (out_f - out_r).abs().max() / out_r.abs().max() < 1e-2
+    for n in g_r:
+        assert (g_f[n] - g_r[n]).abs().max() / g_r[n].abs().max().clamp_min(1e-20) < 2e-2, n
+    assert g_f["patch_embed.proj.weight"].abs().max() > 0
+    odd = []
+    for im in images:
+        buf = torch.zeros(im.size + 1, dtype=torch.uint8, device=DEV)
+        buf[1:].copy_(torch.from_numpy(im).reshape(-1))
+        odd.append(buf[1:].view(im.shape))
+    out_o, g_o = run(frames=odd)
+    assert torch.equal(out_o, out_r) and all(torch.equal(g_o[n], g_r[n]) for n in g_r)
+    with pytest.raises(ValueError, match="either"):
+        tower(hidden_states=pv, grid_thw=grid, frames=frames)
+    with pytest.raises(ValueError, match="does not describe"):
+        tower(frames=frames, grid_thw=torch.tensor([[1, 4, 6]]))
 
 
 # ------------------------------------------------------------------------------------------------ resize
