@@ -194,6 +194,33 @@ def test_trainer_steps_on_gpu():
     assert stats["peak_mb"] >= stats["allocated_mb"] > 0
 
 
+def test_trainer_batched_five_dimensional_pixel_values():
+    """The collated [B, C, T, H, W] input of python/ray/vision.py:732-760: every sample is viewed as consecutive
+    1176-value rows, one grid is broadcast to all samples, and the output comes back as [B, tokens per image, hidden];
+    gradients of a 3-D output arrive in the same shape."""
+    from mi355_vit.trainer import VisionTrainer
+
+    torch.manual_seed(3)
+    px = torch.randn(3, 3, 2, 56, 56)  # 16 rows of 1176 values per sample
+    batches = [{"pixel_values": px, "image_grid_thw": torch.tensor([1, 4, 4]), "sample_index": torch.tensor([5, 6, 7])},
+               {"pixel_values": px.reshape(-1, 1176), "image_grid_thw": torch.tensor([[1, 4, 4]] * 3), "sample_index": torch.tensor([0])}]
+    outs = []
+    for batch in batches:
+        tr = VisionTrainer(_trainer_config(autocast=False), rank=0)
+        tr.build_model()
+        tr.set_data_iterator([batch])
+        tr.initialize_trainer()
+        res = tr.forward_step(0)
+        outs.append(res["vision_embeddings"])
+        if batch["pixel_values"].dim() == 5:
+            assert res["sample_index"] == [5, 6, 7] and tuple(outs[0].shape) == (3, 4, 128)
+            tr.backward_step(torch.ones(3, 4, 128, device=DEV, dtype=torch.bfloat16))
+            assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in tr.model.parameters())
+            with pytest.raises(ValueError, match="doesn't match pixel_values batch dimension"):
+                tr._model_forward({"pixel_values": px.to(DEV), "image_grid_thw": torch.tensor([[1, 4, 4]] * 2, device=DEV)})
+    assert tuple(outs[1].shape) == (1, 12, 128) and torch.equal(outs[0].reshape(1, 12, 128), outs[1])
+
+
 def test_trainer_fifo_and_checkpoint_roundtrip(tmp_path):
     from mi355_vit.trainer import VisionTrainer
 
