@@ -1096,9 +1096,13 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
       __builtin_amdgcn_sched_barrier(0);
     }
     // tile it+2 (requested in iteration it-1) must have landed before any wave reads it in the next iteration; the
-    // loads requested in this iteration (at most five) may stay in flight
-    if (qs + 3 * BQ < L) wait_vmcnt<5>();
-    else wait_vmcnt<0>();
+    // loads requested in this iteration (five by waves 0 and 1, four by the others) may stay in flight
+    if (qs + 3 * BQ < L) {
+      if (wv < 2) wait_vmcnt<5>();
+      else wait_vmcnt<4>();
+    } else {
+      wait_vmcnt<0>();
+    }
     fix_tail(qs + 2 * BQ, (it + 2) & 3);
     __syncthreads();
   }
