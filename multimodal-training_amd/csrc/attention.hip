@@ -548,7 +548,9 @@ __device__ __forceinline__ unsigned pack2(float a, float b) {
 }
 // lanes l and l^16 trade: afterwards a = the pair's value for the lower lane's column, b = for the upper lane's
 __device__ __forceinline__ void swap16(unsigned& a, unsigned& b) {
-  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  const auto r = __builtin_amdgcn_permlane16_swap(a, b, false, false);  // the compiler spaces it from the writes of a and b
+  a = r[0];
+  b = r[1];
 }
 struct BOps {
   bf16x8 lo, hi;  // B operands of the 16x16x32 product for columns l%16 and 16 + l%16 of the 32-column tile
