@@ -15,6 +15,7 @@
 #include "mvit_common.h"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace {
 
@@ -962,6 +963,14 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
     }
     if (wv < 2) lds_direct_4((wv == 0 ? lds_nl0 : lds_nd0) + slot * 256, (unsigned)(min(l, last) * 4), (wv == 0 ? NLSE : NDEL) + qs);
   };
+  auto request_inner_tile = [&](int qs, int slot) {  // the same for a tile of 32 rows inside the segment
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      lds_direct_16(lds_q0 + slot * (XS_TILE * 2) + (2 * wv + j) * 1024, voff_q[j], QS + (int64_t)qs * p.qs_stride);
+      lds_direct_16(lds_do0 + slot * (XS_TILE * 2) + (2 * wv + j) * 1024, voff_do[j], DO + (int64_t)qs * p.do_stride);
+    }
+    if (wv < 2) lds_direct_4((wv == 0 ? lds_nl0 : lds_nd0) + slot * 256, (unsigned)(l < BQ ? l * 4 : (BQ - 1) * 4), (wv == 0 ? NLSE : NDEL) + qs);
+  };
   // statistics of rows past the segment end: probability zero, no contribution
   auto fix_tail = [&](int qs, int slot) {
     if (qs < L && qs + BQ > L && threadIdx.x < BQ && qs + (int)threadIdx.x >= L) {
@@ -1014,11 +1023,16 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
     }
   };
 
-  int it = 0;
-  for (int qs = 0; qs < L; qs += BQ, ++it) {
+  // One step of the loop over tiles.  INNER: tile it+3 lies wholly inside the segment, so its request needs no bounds,
+  // the wait at the end always leaves one tile in flight and no statistics need fixing: the steady state of a long
+  // segment runs without the scalar bookkeeping of the general step, which only the last tiles take.
+  int it = 0, qs = 0;
+  auto step = [&](auto inner_tag) {
+    constexpr bool INNER = decltype(inner_tag)::value;
     const int b0 = it & 3, b1 = (it + 1) & 3, b3 = (it + 3) & 3;
     // tile it+3 is requested into the slot that tile it-1 left (every wave is past the barrier that ended iteration it-1)
-    request_tile(qs + 3 * BQ, b3);
+    if constexpr (INNER) request_inner_tile(qs + 3 * BQ, b3);
+    else request_tile(qs + 3 * BQ, b3);
     // ---- phase 1: score products of key group 0; the transposed left factors that phase 3 needs are read from LDS
     // between the MFMAs
     bf16x8 qt[ND], dt_[ND];
@@ -1099,15 +1113,17 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
     }
     // tile it+2 (requested in iteration it-1) must have landed before any wave reads it in the next iteration; the
     // loads requested in this iteration (five by waves 0 and 1, four by the others) may stay in flight
-    if (qs + 3 * BQ < L) {
+    if (INNER || qs + 3 * BQ < L) {
       if (wv < 2) wait_vmcnt<5>();
       else wait_vmcnt<4>();
     } else {
       wait_vmcnt<0>();
     }
-    fix_tail(qs + 2 * BQ, (it + 2) & 3);
+    if constexpr (!INNER) fix_tail(qs + 2 * BQ, (it + 2) & 3);
     __syncthreads();
-  }
+  };
+  for (; qs + 4 * BQ <= L; qs += BQ, ++it) step(std::true_type{});
+  for (; qs < L; qs += BQ, ++it) step(std::false_type{});
 
   bf16_t* DK = static_cast<bf16_t*>(p.dk) + (int64_t)s0 * p.dk_stride + (int64_t)h * HD;
   bf16_t* DV = static_cast<bf16_t*>(p.dv) + (int64_t)s0 * p.dv_stride + (int64_t)h * HD;
