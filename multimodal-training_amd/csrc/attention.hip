@@ -890,11 +890,8 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
   static_assert(ND == 5, "the hand-placed instruction order below is laid out for head_dim 80");
   using G = Geo<ND>;
   constexpr int HD = G::HD, BQ = 32, NT = 256, RING = 4;
-  // one array for both streamed tensors: a fragment's address in the dO tile is its address in the Q tile plus a
-  // constant that fits the instruction's offset field, so one address computation serves both
-  __shared__ __attribute__((aligned(1024))) bf16_t lds_qd[2 * RING][XS_TILE];
-  bf16_t (*const lds_q)[XS_TILE] = lds_qd;
-  bf16_t (*const lds_do)[XS_TILE] = lds_qd + RING;
+  __shared__ __attribute__((aligned(1024))) bf16_t lds_q[RING][XS_TILE];
+  __shared__ __attribute__((aligned(1024))) bf16_t lds_do[RING][XS_TILE];
   __shared__ __attribute__((aligned(256))) float lds_nlse[RING][64];  // - lse * log2(e) per query of the tile (32 used)
   __shared__ __attribute__((aligned(256))) float lds_ndel[RING][64];  // - delta
   __shared__ __attribute__((aligned(16))) float lds_fix[NT * 4];
@@ -1432,7 +1429,9 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_wide(const AttnParams p) {
   static_assert(ND == 5, "the hand-placed instruction order below is laid out for head_dim 80");
   using G = Geo<ND>;
   constexpr int HD = G::HD, BK = 32, NT = 256, RING = 4;
-  __shared__ __attribute__((aligned(1024))) bf16_t lds_kv[2 * RING][XS_TILE];  // one array: see attn_bwd_dkdv_wide
+  // one array for both streamed tensors: a fragment's address in the V tile is its address in the K tile plus a
+  // constant that fits the instruction's offset field, so one address computation serves both
+  __shared__ __attribute__((aligned(1024))) bf16_t lds_kv[2 * RING][XS_TILE];
   bf16_t (*const lds_k)[XS_TILE] = lds_kv;
   bf16_t (*const lds_v)[XS_TILE] = lds_kv + RING;
   __shared__ __attribute__((aligned(16))) float lds_fix[NT * 4];
