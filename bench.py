@@ -199,6 +199,14 @@ def handoff_leg(n_vision: int, hidden: int, dtype, iters: int = 20):
         text.grad = None
         return extract_vision_grad(leaf)
 
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            fn()
+        torch.cuda.synchronize()
+        return 1000.0 * (time.perf_counter() - t0) / iters
 
     assert torch.equal(ours(), reference_calls())
     ours_ms, ref_ms = timed(ours), timed(reference_calls)
