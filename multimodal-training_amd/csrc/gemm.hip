@@ -1238,15 +1238,39 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
 }
 
 // C[m, n] = sum over slices of the fp32 partial tiles (fixed order, so the result is reproducible).
-template <typename TO>
+// VEC: four consecutive columns per thread (N, ldc and the pointers allow 16-byte accesses).
+template <typename TO, bool VEC>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, int split_k, int64_t M, int64_t N,
                                                             TO* __restrict__ C, int64_t ldc) {
   const int64_t total = M * N;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-    float s = 0.f;
-    for (int k = 0; k < split_k; ++k) s += ws[(int64_t)k * total + i];
-    C[(i / N) * ldc + (i % N)] = from_f32<TO>(s);
+  if constexpr (VEC) {
+    const int64_t quads = total / 4, nq = N / 4;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < quads; i += (int64_t)gridDim.x * 256) {
+      f32x4 s = {0.f, 0.f, 0.f, 0.f};  // the same sum, from the same zero, as the scalar form
+      for (int k = 0; k < split_k; ++k) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(ws + (int64_t)k * total + 4 * i);
+        s = f32x4{s[0] + v[0], s[1] + v[1], s[2] + v[2], s[3] + v[3]};
+      }
+      TO* c = C + (i / nq) * ldc + (i % nq) * 4;
+      if constexpr (sizeof(TO) == 2) *reinterpret_cast<bf16x4*>(c) = bf16x4{(bf16_t)s[0], (bf16_t)s[1], (bf16_t)s[2], (bf16_t)s[3]};
+      else *reinterpret_cast<f32x4*>(c) = s;
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+      float s = 0.f;
+      for (int k = 0; k < split_k; ++k) s += ws[(int64_t)k * total + i];
+      C[(i / N) * ldc + (i % N)] = from_f32<TO>(s);
+    }
   }
+}
+template <typename TO>
+void launch_splitk_reduce(const GemmParams& p, hipStream_t stream) {
+  const int64_t elems = p.M * p.N;
+  const bool vec = p.N % 4 == 0 && p.ldc % 4 == 0 && mvit_aligned16(p.workspace) && (reinterpret_cast<uintptr_t>(p.C) % (4 * sizeof(TO))) == 0;
+  const int64_t items = vec ? elems / 4 : elems;
+  const int rgrid = (int)((items + 255) / 256 < 8192 ? (items + 255) / 256 : 8192);
+  if (vec) hipLaunchKernelGGL((splitk_reduce_kernel<TO, true>), rgrid, 256, 0, stream, p.workspace, p.split_k, p.M, p.N, static_cast<TO*>(p.C), p.ldc);
+  else hipLaunchKernelGGL((splitk_reduce_kernel<TO, false>), rgrid, 256, 0, stream, p.workspace, p.split_k, p.M, p.N, static_cast<TO*>(p.C), p.ldc);
 }
 
 template <typename T, typename TO, bool TA, bool TB, int EPI, int VAR>
@@ -1271,9 +1295,7 @@ int launch(const GemmParams& p, hipStream_t stream) {
   hipLaunchKernelGGL(kern, grid, W::NTHREADS, lds, stream, p);
   MVIT_CHECK_LAUNCH("gemm");
   if (p.split_k > 1) {
-    const int64_t elems = p.M * p.N;
-    const int rgrid = (int)((elems + 255) / 256 < 8192 ? (elems + 255) / 256 : 8192);
-    hipLaunchKernelGGL((splitk_reduce_kernel<TO>), rgrid, 256, 0, stream, p.workspace, p.split_k, p.M, p.N, static_cast<TO*>(p.C), p.ldc);
+    launch_splitk_reduce<TO>(p, stream);
     MVIT_CHECK_LAUNCH("gemm split-k reduce");
   }
   return MVIT_OK;
@@ -1308,9 +1330,7 @@ int launch_dl(const GemmParams& p, hipStream_t stream) {
   hipLaunchKernelGGL(kern, grid, D::NTHREADS, lds, stream, p);
   MVIT_CHECK_LAUNCH("gemm");
   if (p.split_k > 1) {
-    const int64_t elems = p.M * p.N;
-    const int rgrid = (int)((elems + 255) / 256 < 8192 ? (elems + 255) / 256 : 8192);
-    hipLaunchKernelGGL((splitk_reduce_kernel<TO>), rgrid, 256, 0, stream, p.workspace, p.split_k, p.M, p.N, static_cast<TO*>(p.C), p.ldc);
+    launch_splitk_reduce<TO>(p, stream);
     MVIT_CHECK_LAUNCH("gemm split-k reduce");
   }
   return MVIT_OK;
