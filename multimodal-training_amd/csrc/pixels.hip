@@ -215,6 +215,83 @@ __global__ __launch_bounds__(256) void resample_rows_lds_kernel(const uint8_t* _
   }
 }
 
+// The horizontal pass again, for windows of at most RESAMPLE_KMAX taps: a work-group owns 256 consecutive output
+// coordinates and a strip of rows.  A thread keeps its coordinate's window and weights in registers for the whole strip
+// (they are the same for every row, and fetching them per row was most of the row kernel's time); per row the
+// work-group stages just the input bytes its 256 windows cover (two LDS buffers, one barrier per row) and every thread
+// makes one pixel.  A work-group whose windows cover more than the LDS buffer (windows are the caller's) reads its taps
+// from global memory instead.
+constexpr int RESAMPLE_KMAX = 16, RESAMPLE_SPAN_BYTES = 8 * 1024;
+__global__ __launch_bounds__(256) void resample_cols_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int64_t outer,
+                                                            int64_t in_len, int64_t out_len, int inner, const int32_t* __restrict__ bounds,
+                                                            const int32_t* __restrict__ kk, int ksize, int rows_per_group) {
+  __shared__ __attribute__((aligned(16))) uint8_t buf[2][RESAMPLE_SPAN_BYTES + 8];
+  const int64_t row_in = in_len * inner, row_out = out_len * inner;
+  const uint8_t* src_end = src + outer * row_in;
+  const int x_first = blockIdx.x * 256, x_last = min(x_first + 255, (int)out_len - 1);
+  const bool mine = x_first + (int)threadIdx.x <= x_last;
+  const int x = mine ? x_first + (int)threadIdx.x : x_last;
+  const int xmin = bounds[2 * x], n = bounds[2 * x + 1];
+  int k[RESAMPLE_KMAX];
+#pragma unroll
+  for (int t = 0; t < RESAMPLE_KMAX; ++t) k[t] = t < n ? kk[(int64_t)x * ksize + t] : 0;
+  // bytes of a row that the work-group's windows cover (window starts and ends do not decrease with the coordinate
+  // for a resampling; anything else shows up as a span that does not fit and takes the global path)
+  int lo = bounds[2 * x_first] * inner, hi = (bounds[2 * x_last] + bounds[2 * x_last + 1]) * inner;
+  bool fits = hi - lo + 4 <= RESAMPLE_SPAN_BYTES && xmin * inner >= lo && (xmin + n) * inner <= hi;
+  fits = __syncthreads_and(fits);
+  const int64_t o_begin = (int64_t)blockIdx.y * rows_per_group, o_end = min(o_begin + rows_per_group, outer);
+  for (int64_t o = o_begin; o < o_end; ++o) {
+    int acc[RESAMPLE_MAX_CHANNELS];
+#pragma unroll
+    for (int c = 0; c < RESAMPLE_MAX_CHANNELS; ++c) acc[c] = 1 << (RESAMPLE_PRECISION_BITS - 1);
+    if (fits) {
+      const uint8_t* b = src + o * row_in + lo;
+      const int lead = (int)((uintptr_t)b & 3);
+      const uint8_t* a = b - lead;
+      const int words = (lead + (hi - lo) + 3) / 4;
+      uint8_t* stage = buf[o & 1];
+      for (int j = threadIdx.x; j < words; j += 256) {
+        const uint8_t* g = a + 4 * j;
+        unsigned w;
+        if (g >= src && g + 4 <= src_end) {
+          w = *reinterpret_cast<const unsigned*>(g);
+        } else {  // first / last word of the array: only the bytes that belong to it
+          w = 0;
+          for (int e = 0; e < 4; ++e)
+            if (g + e >= src && g + e < src_end) w |= (unsigned)g[e] << (8 * e);
+        }
+        *reinterpret_cast<unsigned*>(stage + 4 * j) = w;
+      }
+      __syncthreads();  // also: every thread is done with the buffer of two rows ago
+      const uint8_t* px = stage + lead + (xmin * inner - lo);
+#pragma unroll
+      for (int t = 0; t < RESAMPLE_KMAX; ++t) {
+        if (t >= ksize) break;
+        const uint8_t* q = px + max(min(t, n - 1), 0) * inner;  // taps past the window have weight 0 and re-read its last one
+#pragma unroll
+        for (int c = 0; c < RESAMPLE_MAX_CHANNELS; ++c)
+          if (c < inner) acc[c] += (int)q[c] * k[t];
+      }
+    } else {
+      const uint8_t* px = src + o * row_in + (int64_t)xmin * inner;
+#pragma unroll
+      for (int t = 0; t < RESAMPLE_KMAX; ++t) {
+        if (t >= n) break;
+#pragma unroll
+        for (int c = 0; c < RESAMPLE_MAX_CHANNELS; ++c)
+          if (c < inner) acc[c] += (int)px[t * inner + c] * k[t];
+      }
+    }
+    if (mine) {
+      uint8_t* d = dst + o * row_out + (int64_t)x * inner;
+#pragma unroll
+      for (int c = 0; c < RESAMPLE_MAX_CHANNELS; ++c)
+        if (c < inner) d[c] = (uint8_t)clip8(acc[c]);
+    }
+  }
+}
+
 extern "C" {
 
 int mvit_patchify(const mvit_image* images, int n_images, int64_t total_rows, void* out, double rescale, float mean_r,
@@ -248,7 +325,12 @@ int mvit_resample_u8(const uint8_t* src, uint8_t* dst, int64_t outer, int64_t in
   const int64_t quads = (out_len * inner + 3) / 4, total = outer * quads;
   const unsigned grid = (unsigned)((total + 255) / 256 < 65535 * 16 ? (total + 255) / 256 : 65535 * 16);
   const bool wide = inner % 4 == 0 && ((uintptr_t)src % 4 == 0) && ((uintptr_t)dst % 4 == 0);
-  if (!wide && inner <= RESAMPLE_MAX_CHANNELS && in_len * inner + 4 <= RESAMPLE_LDS_BYTES) {
+  if (!wide && inner <= RESAMPLE_MAX_CHANNELS && ksize <= RESAMPLE_KMAX) {
+    const int rows_per_group = 32;
+    const dim3 g((unsigned)((out_len + 255) / 256), (unsigned)((outer + rows_per_group - 1) / rows_per_group));
+    MVIT_REQUIRE(g.y <= 65535, "resample_u8: outer=%lld too large for a short inner dimension", (long long)outer);
+    hipLaunchKernelGGL(resample_cols_kernel, g, 256, 0, s, src, dst, outer, in_len, out_len, (int)inner, bounds, kk, ksize, rows_per_group);
+  } else if (!wide && inner <= RESAMPLE_MAX_CHANNELS && in_len * inner + 4 <= RESAMPLE_LDS_BYTES) {
     const unsigned rows = (unsigned)(outer < 65535 * 16 ? outer : 65535 * 16);
     hipLaunchKernelGGL(resample_rows_lds_kernel, dim3(rows), 256, 0, s, src, dst, outer, in_len, out_len, (int)inner, bounds, kk, ksize);
   } else if (wide) hipLaunchKernelGGL((resample_pass_kernel<true>), dim3(grid), 256, 0, s, src, dst, outer, in_len, out_len, inner, bounds, kk, ksize);

@@ -350,7 +350,9 @@ def test_resize_bit_exact_against_oracle_and_pillow(name):
 
     rng = np.random.default_rng(11)
     cases = [(1, 37, 53, 28, 56), (1, 100, 80, 56, 56), (2, 28, 28, 112, 84), (1, 5, 7, 28, 28), (3, 64, 64, 64, 32), (1, 64, 60, 28, 60),
-             (1, 211, 157, 140, 196), (1, 33, 1, 28, 28), (1, 90, 61, 45, 33), (1, 300, 200, 299, 201)]
+             (1, 211, 157, 140, 196), (1, 33, 1, 28, 28), (1, 90, 61, 45, 33), (1, 300, 200, 299, 201),
+             (1, 40, 400, 28, 56),    # windows of 17 / 31 taps: beyond what the column kernel keeps in registers
+             (1, 70, 900, 28, 700)]   # three column blocks of 256 output pixels, 70 rows = three row strips
     try:
         from PIL import Image
         filt = {"bilinear": Image.Resampling.BILINEAR, "bicubic": Image.Resampling.BICUBIC}[name]
@@ -365,6 +367,37 @@ def test_resize_bit_exact_against_oracle_and_pillow(name):
             assert np.array_equal(got[i], ro.pil_resize(img[i], oh, ow, name)), (f, h, w, oh, ow, i)
             if Image is not None:
                 assert np.array_equal(got[i], np.asarray(Image.fromarray(img[i]).resize((ow, oh), filt)))
+
+
+def test_resample_pass_with_windows_of_the_callers_own():
+    """mvit_resample_u8 takes any windows, not only those of a resize: a mirrored pass (output x reads the inputs
+    around in_len - 1 - x, so window starts decrease with x and no LDS span covers a work-group's windows) against numpy."""
+    import ctypes as C
+
+    from mi355_vit import _lib
+
+    _announce("resample with mirrored windows")
+    rng = np.random.default_rng(21)
+    outer, in_len, out_len, inner, ksize = 37, 300, 280, 3, 3
+    src = rng.integers(0, 256, (outer, in_len, inner), dtype=np.uint8)
+    bounds = np.zeros((out_len, 2), dtype=np.int32)
+    kk = np.zeros((out_len, ksize), dtype=np.int32)
+    for x in range(out_len):
+        c = in_len - 2 - x
+        bounds[x] = (c - 1, 3) if c >= 1 else (0, 2)
+        kk[x, : bounds[x, 1]] = ((1 << 20), (1 << 21), (1 << 20)) if c >= 1 else ((1 << 21), (1 << 21))
+    ref = np.empty((outer, out_len, inner), dtype=np.uint8)
+    for x in range(out_len):
+        lo, n = bounds[x]
+        acc = (1 << 21) + (src[:, lo : lo + n, :].astype(np.int64) * kk[x, :n, None]).sum(axis=1)
+        ref[:, x, :] = np.clip(acc >> 22, 0, 255)
+    d_src, d_b, d_k = (torch.from_numpy(a).to(DEV) for a in (src, bounds, kk))
+    d_dst = torch.zeros(outer, out_len, inner, dtype=torch.uint8, device=DEV)
+    rc = _lib.load().mvit_resample_u8(d_src.data_ptr(), d_dst.data_ptr(), outer, in_len, out_len, inner, d_b.data_ptr(), d_k.data_ptr(), ksize,
+                                      torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "mvit_resample_u8")
+    torch.cuda.synchronize()
+    assert np.array_equal(d_dst.cpu().numpy(), ref)
 
 
 def test_resize_large_image_against_pillow_and_the_whole_input_chain():
