@@ -969,7 +969,9 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
       lds_direct_16(lds_q0 + slot * (XS_TILE * 2) + (2 * wv + j) * 1024, voff_q[j], QS + (int64_t)qs * p.qs_stride);
       lds_direct_16(lds_do0 + slot * (XS_TILE * 2) + (2 * wv + j) * 1024, voff_do[j], DO + (int64_t)qs * p.do_stride);
     }
-    if (wv < 2) lds_direct_4((wv == 0 ? lds_nl0 : lds_nd0) + slot * 256, (unsigned)(l < BQ ? l * 4 : (BQ - 1) * 4), (wv == 0 ? NLSE : NDEL) + qs);
+    // every wave fetches one array of statistics (waves 2 and 3 the same bytes as 0 and 1): five loads per wave and
+    // tile, so the wait at the end of the step is the same instruction for all of them
+    lds_direct_4(((wv & 1) == 0 ? lds_nl0 : lds_nd0) + slot * 256, (unsigned)(l < BQ ? l * 4 : (BQ - 1) * 4), ((wv & 1) == 0 ? NLSE : NDEL) + qs);
   };
   // statistics of rows past the segment end: probability zero, no contribution
   auto fix_tail = [&](int qs, int slot) {
@@ -1113,7 +1115,9 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
     }
     // tile it+2 (requested in iteration it-1) must have landed before any wave reads it in the next iteration; the
     // loads requested in this iteration (five by waves 0 and 1, four by the others) may stay in flight
-    if (INNER || qs + 3 * BQ < L) {
+    if constexpr (INNER) {
+      wait_vmcnt<5>();
+    } else if (qs + 3 * BQ < L) {
       if (wv < 2) wait_vmcnt<5>();
       else wait_vmcnt<4>();
     } else {
