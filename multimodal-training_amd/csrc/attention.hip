@@ -2253,6 +2253,7 @@ int check_common(const char* who, const int32_t* cu, int n_seg, int max_seqlen, 
   const int vec = dtype == MVIT_BF16 ? 8 : 1;
   for (int64_t st : strides)
     MVIT_REQUIRE(st >= (int64_t)nheads * head_dim && st % vec == 0, "%s: row stride %lld must cover %d heads and be a multiple of %d", who, (long long)st, nheads, vec);
+  if (n_seg == 0 || max_seqlen == 0 || total == 0) return MVIT_OK;  // nothing to do: empty tensors have no address to check
   for (const void* q : ptrs) MVIT_REQUIRE(q && mvit_aligned16(q), "%s: null or unaligned pointer", who);
   return MVIT_OK;
 }

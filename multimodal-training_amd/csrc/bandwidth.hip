@@ -398,9 +398,9 @@ extern "C" {
 
 int mvit_rmsnorm_fwd(const void* x, const void* w, void* y, float* rstd, int64_t rows, int64_t cols, float eps,
                      int dtype, mvit_stream_t stream) {
-  MVIT_REQUIRE(x && w && y && rstd, "rmsnorm_fwd: null pointer");
   MVIT_REQUIRE(rows >= 0 && cols > 0 && cols < (1 << 24), "rmsnorm_fwd: bad shape %lld x %lld", (long long)rows, (long long)cols);
   if (rows == 0) return MVIT_OK;
+  MVIT_REQUIRE(x && w && y && rstd, "rmsnorm_fwd: null pointer");
   const int grid = clamp_grid((rows + 3) / 4, 8192);
   if (dtype == MVIT_BF16) {
     const bool vec = cols % 8 == 0 && mvit_aligned16(x) && mvit_aligned16(y) && mvit_aligned16(w);
@@ -423,7 +423,7 @@ int mvit_rmsnorm_fwd(const void* x, const void* w, void* y, float* rstd, int64_t
 
 int mvit_rmsnorm_bwd(const void* dy, const void* x, const void* w, const float* rstd, const void* dx_add, void* dx,
                      float* dw_partial, int n_partial, int64_t rows, int64_t cols, int dtype, mvit_stream_t stream) {
-  MVIT_REQUIRE(dy && x && w && rstd && dx && dw_partial, "rmsnorm_bwd: null pointer");
+  MVIT_REQUIRE(dw_partial && w && (rows == 0 || (dy && x && rstd && dx)), "rmsnorm_bwd: null pointer");  // no rows: only the partial sums are written (zeros)
   MVIT_REQUIRE(rows >= 0 && cols > 0 && n_partial > 0, "rmsnorm_bwd: bad shape");
   const size_t lds = 4 * (size_t)cols * sizeof(float);
   MVIT_REQUIRE(lds <= 160 * 1024, "rmsnorm_bwd: cols %lld needs %zu B of LDS (> 160 KiB)", (long long)cols, lds);
@@ -469,7 +469,7 @@ int mvit_reduce_partials(const float* partial, int n_partial, int64_t cols, void
 }
 
 int mvit_colsum(const void* x, int64_t ld, int64_t rows, int64_t cols, float* partial, int n_partial, int dtype, mvit_stream_t stream) {
-  MVIT_REQUIRE(x && partial && n_partial > 0 && n_partial <= 65535 && cols > 0 && rows >= 0 && ld >= cols, "colsum: bad arguments");
+  MVIT_REQUIRE((x || rows == 0) && partial && n_partial > 0 && n_partial <= 65535 && cols > 0 && rows >= 0 && ld >= cols, "colsum: bad arguments");
   MVIT_REQUIRE(dtype == MVIT_BF16 || dtype == MVIT_F32, "colsum: dtype %d", dtype);
   const int vec = dtype == MVIT_BF16 ? 8 : 4;
   if (cols % vec == 0 && ld % vec == 0 && mvit_aligned16(x)) {
@@ -491,10 +491,10 @@ int mvit_colsum(const void* x, int64_t ld, int64_t rows, int64_t cols, float* pa
 
 int mvit_rope(void* x, const float* cosb, const float* sinb, int64_t rows, int nheads, int head_dim, int64_t row_stride,
               int backward, int dtype, mvit_stream_t stream) {
-  MVIT_REQUIRE(x && cosb && sinb, "rope: null pointer");
   MVIT_REQUIRE(rows >= 0 && nheads > 0 && head_dim > 0 && head_dim % 2 == 0 && row_stride >= (int64_t)nheads * head_dim,
                "rope: bad shape rows=%lld heads=%d head_dim=%d stride=%lld", (long long)rows, nheads, head_dim, (long long)row_stride);
   if (rows == 0) return MVIT_OK;
+  MVIT_REQUIRE(x && cosb && sinb, "rope: null pointer");
   const int half = head_dim / 2;
   const int64_t work_scalar = rows * nheads * half;
   if (dtype == MVIT_BF16) {
@@ -521,9 +521,9 @@ int mvit_rope(void* x, const float* cosb, const float* sinb, int64_t rows, int n
 }
 
 int mvit_gather_rows(const void* src, const int64_t* index, void* dst, int64_t n_rows, int64_t row_bytes, mvit_stream_t stream) {
-  MVIT_REQUIRE(src && index && dst, "gather_rows: null pointer");
   MVIT_REQUIRE(n_rows >= 0 && row_bytes > 0 && row_bytes % 2 == 0, "gather_rows: row_bytes %lld must be a positive multiple of 2", (long long)row_bytes);
   if (n_rows == 0) return MVIT_OK;
+  MVIT_REQUIRE(src && index && dst, "gather_rows: null pointer");
   const unsigned gy = (unsigned)clamp_grid(n_rows, 65535);
   if (row_bytes % 16 == 0 && mvit_aligned16(src) && mvit_aligned16(dst)) {
     const int64_t words = row_bytes / 16;
@@ -543,9 +543,9 @@ int mvit_gather_rows(const void* src, const int64_t* index, void* dst, int64_t n
 }
 
 int mvit_segment_copy(const void* src, void* dst, const int64_t* desc, int64_t nseg, int64_t max_seg_rows, int64_t row_bytes, mvit_stream_t stream) {
-  MVIT_REQUIRE(src && dst && desc, "segment_copy: null pointer");
   MVIT_REQUIRE(nseg >= 0 && nseg <= 65535 && row_bytes > 0 && row_bytes % 2 == 0, "segment_copy: bad nseg/row_bytes");
   if (nseg == 0 || max_seg_rows <= 0) return MVIT_OK;
+  MVIT_REQUIRE(src && dst && desc, "segment_copy: null pointer");
   const unsigned gy = (unsigned)clamp_grid(max_seg_rows, 4096);
   if (row_bytes % 16 == 0 && mvit_aligned16(src) && mvit_aligned16(dst)) {
     const int64_t words = row_bytes / 16;
@@ -566,10 +566,10 @@ int mvit_segment_copy(const void* src, void* dst, const int64_t* desc, int64_t n
 
 int mvit_pad_pack(const void* pack, void* padded, uint8_t* mask, const int64_t* lens, const int64_t* offsets, int64_t batch,
                   int64_t pad_len, int64_t row_elems, int elem_size, uint32_t pad_bits, mvit_stream_t stream) {
-  MVIT_REQUIRE(padded && mask && lens && offsets, "pad_pack: null pointer");
   MVIT_REQUIRE(batch >= 0 && batch <= 65535 && pad_len >= 0 && row_elems > 0, "pad_pack: bad shape");
   MVIT_REQUIRE(elem_size == 2 || elem_size == 4, "pad_pack: elem_size %d", elem_size);
   if (batch == 0 || pad_len == 0) return MVIT_OK;
+  MVIT_REQUIRE(padded && mask && lens && offsets, "pad_pack: null pointer");
   dim3 grid((unsigned)clamp_grid((row_elems + 255) / 256, 64), (unsigned)clamp_grid(pad_len, 4096), (unsigned)batch);
   if (elem_size == 2)
     hipLaunchKernelGGL((pad_pack_kernel<uint16_t>), grid, 256, 0, S_(stream), (const uint16_t*)pack, (uint16_t*)padded, mask, lens, offsets, pad_len, row_elems, (uint16_t)pad_bits);
@@ -581,8 +581,9 @@ int mvit_pad_pack(const void* pack, void* padded, uint8_t* mask, const int64_t* 
 
 int mvit_cast2d(const void* src, int64_t src_ld, int src_dtype, void* dst, int64_t dst_ld, int dst_dtype, int64_t rows,
                 int64_t cols, mvit_stream_t stream) {
-  MVIT_REQUIRE(src && dst && rows >= 0 && cols >= 0 && src_ld >= cols && dst_ld >= cols, "cast2d: bad arguments");
+  MVIT_REQUIRE(rows >= 0 && cols >= 0 && src_ld >= cols && dst_ld >= cols, "cast2d: bad arguments");
   if (rows == 0 || cols == 0) return MVIT_OK;
+  MVIT_REQUIRE(src && dst, "cast2d: null pointer");
   dim3 grid((unsigned)clamp_grid((cols + 255) / 256, 256), (unsigned)clamp_grid(rows, 16384));
   hipStream_t s = S_(stream);
   if (src_dtype == MVIT_F32 && dst_dtype == MVIT_BF16)
@@ -601,7 +602,7 @@ int mvit_cast2d(const void* src, int64_t src_ld, int src_dtype, void* dst, int64
 
 int mvit_image_token_ranks(const int64_t* input_ids, const int64_t* labels, int64_t n_tokens, int64_t image_token_id,
                            int64_t ignore_label, int32_t* rank, int64_t* positions, int64_t* counts, mvit_stream_t stream) {
-  MVIT_REQUIRE(input_ids && rank && positions && counts, "image_token_ranks: null pointer");
+  MVIT_REQUIRE(counts && (n_tokens == 0 || (input_ids && rank && positions)), "image_token_ranks: null pointer");  // no tokens: only the counts are written (zeros)
   MVIT_REQUIRE(n_tokens >= 0 && n_tokens <= 0x7fffffffLL, "image_token_ranks: n_tokens %lld out of range", (long long)n_tokens);
   hipLaunchKernelGGL(image_token_ranks_kernel, dim3(1), 1024, 0, S_(stream), input_ids, labels, n_tokens, image_token_id, ignore_label,
                      rank, positions, counts);
@@ -611,9 +612,9 @@ int mvit_image_token_ranks(const int64_t* input_ids, const int64_t* labels, int6
 
 int mvit_merge_rows(const void* embeds, const void* vision, const int32_t* rank, void* merged, int64_t n_tokens, int64_t n_vision,
                     int64_t row_bytes, mvit_stream_t stream) {
-  MVIT_REQUIRE(embeds && rank && merged, "merge_rows: null pointer");
   MVIT_REQUIRE(n_tokens >= 0 && n_vision >= 0 && row_bytes > 0 && row_bytes % 2 == 0, "merge_rows: bad sizes (row_bytes %lld)", (long long)row_bytes);
   if (n_tokens == 0) return MVIT_OK;
+  MVIT_REQUIRE(embeds && rank && merged, "merge_rows: null pointer");
   const unsigned gy = (unsigned)clamp_grid(n_tokens, 65535);
   const bool al = mvit_aligned16(embeds) && mvit_aligned16(merged) && (vision == nullptr || mvit_aligned16(vision));
   if (row_bytes % 16 == 0 && al) {

@@ -1472,9 +1472,9 @@ extern "C" int mvit_patch_embed_frames(const mvit_image* images, int n_images, i
 
 extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
   MVIT_REQUIRE(a, "gemm: null args");
-  MVIT_REQUIRE(a->A && a->B && a->C, "gemm: null operand");
   MVIT_REQUIRE(a->M >= 0 && a->N > 0 && a->K > 0, "gemm: bad shape M=%lld N=%lld K=%lld", (long long)a->M, (long long)a->N, (long long)a->K);
   if (a->M == 0) return MVIT_OK;
+  MVIT_REQUIRE(a->A && a->B && a->C, "gemm: null operand");
   const int vec = a->dtype == MVIT_BF16 ? 8 : 4;
   MVIT_REQUIRE(a->dtype == MVIT_BF16 || a->dtype == MVIT_F32, "gemm: dtype %d", a->dtype);
   MVIT_REQUIRE(a->out_dtype == MVIT_BF16 || a->out_dtype == MVIT_F32, "gemm: out_dtype %d", a->out_dtype);
