@@ -85,6 +85,25 @@ def test_small_ragged_tower_bf16_parity(checkpoint):
     assert worst[0] < 2e-2, worst
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 2e-2)])
+def test_smallest_images_parity(dtype, tol):
+    """The smallest inputs the model takes: one 28 x 28 image (4 patches, one merged token: every GEMM has 4 rows, every
+    attention segment 4 tokens) alone and beside a 2-frame video of the same size and a 28 x 56 image, against the oracle."""
+    kw = dict(depth=2, hidden_size=256, intermediate_size=300, num_heads=8, out_hidden_size=128, fullatt_block_indexes=[1])
+    for grid in (torch.tensor([[1, 2, 2]]), torch.tensor([[1, 2, 2], [2, 2, 2], [1, 2, 4]])):
+        print(f"[case] smallest images {grid.tolist()} {dtype}", flush=True)
+        model = _build(kw, 2, dtype)
+        g = torch.Generator().manual_seed(4)
+        S = int((grid[:, 0] * grid[:, 1] * grid[:, 2]).sum())
+        pixels = torch.randn(S, 1176, generator=g).to(dtype)
+        gout = torch.randn(S // 4, 128, generator=g).to(dtype)
+        ref_out, ref_grads = _oracle_run(copy.deepcopy(model), kw, pixels, grid, gout)
+        out, grads = _run_gpu(model, pixels, grid, gout)
+        assert tuple(out.shape) == (S // 4, 128) and max_rel_err(out, ref_out) < tol
+        worst = max((max_rel_err(grads[k], ref_grads[k]), k) for k in ref_grads)
+        assert worst[0] < tol, worst
+
+
 def test_checkpointing_gives_identical_gradients():
     kw = dict(depth=2, hidden_size=256, intermediate_size=300, num_heads=8, out_hidden_size=256, window_size=56, fullatt_block_indexes=[1])
     g = torch.Generator().manual_seed(3)
