@@ -384,6 +384,8 @@ def _attn_case(dtype, seglens, H, d, seed=0, qkv_packed=True):
         ([100, 60], 8, 32),
         ([129], 2, 64),
         ([96, 200], 2, 128),
+        ([65, 128, 127], 2, 80),  # either side of the 64- and 128-token kernel choices
+        ([511, 2], 2, 80),  # one token below the long-segment kernels
         # long segments (the 64-rows-per-wave backward kernels): tile multiples, tails of 1 / 31 / 33 rows, short
         # segments riding in the same launch
         ([512], 2, 80),
