@@ -142,6 +142,33 @@ def test_split_gather_bit_exact(dtype, sp):
         assert sum(m.total_local_len for m in metas) == S
 
 
+def test_split_gather_with_empty_rank_shares():
+    """Samples shorter than the sequence-parallel degree (4-patch images, sp = 8): some ranks receive nothing from a sample,
+    some nothing at all; packs of zero rows travel through split, pad / unpad and the re-interleave like any other."""
+    from mi355_vit import sequence_parallel_utils as spu
+
+    for lengths, sp, some_rank_empty in (([4, 4, 16, 4], 8, False), ([4, 4, 16, 4], 5, False), ([4, 2, 4], 8, True)):
+        S = sum(lengths)
+        x = _rand((S, 64), torch.bfloat16, 7)
+        xg = x.to(DEV)
+        _announce(f"split/gather with empty shares lengths={lengths} sp={sp}")
+        packs, metas = [], []
+        for r in range(sp):
+            pk, meta = spu.split_pack_by_sp(xg, lengths, r, sp)
+            ref = sp_oracle.split_rows(x.view(torch.int16).numpy(), lengths, r, sp, None)
+            assert pk.shape[0] == ref.shape[0] and np.array_equal(pk.cpu().view(torch.int16).numpy().reshape(ref.shape), ref)
+            padded, mask = spu.pad_pack_to_batch(pk, meta, pad_value=-999.0, enforce_min_pad=1)
+            assert padded.shape[:2] == (len(lengths), max(1, meta.max_local_len)) and mask.sum(dim=1).tolist() == list(meta.local_lengths)
+            back, _ = spu.unpad_batch_to_pack(padded, mask)
+            assert torch.equal(back.view(torch.int16), pk.view(torch.int16))
+            packs.append(pk)
+            metas.append(meta)
+        assert any(0 in m.local_lengths for m in metas)
+        assert any(m.total_local_len == 0 for m in metas) == some_rank_empty
+        rebuilt = spu.gather_rank_packs(packs, [m.local_lengths for m in metas])
+        assert torch.equal(rebuilt.cpu().view(torch.uint8), x.view(torch.uint8))
+
+
 def test_split_gather_sp4_real_shape():
     """Five square images with sides drawn from the multiples of 28 in [448, 3584] (seed 2), hidden 1280, bf16,
     split into 4 sequence-parallel shards (token cuts and window-aligned cuts) and gathered back: bit-exact."""
