@@ -122,7 +122,8 @@ enum {
   MVIT_EPI_BIAS = 1,       /* C = acc + bias[n]                                               */
   MVIT_EPI_BIAS_RES = 2,   /* C = acc + bias[n] + R[m,n]                                      */
   MVIT_EPI_BIAS_GELU = 3,  /* aux = acc + bias[n];  C = gelu_erf(aux)                         */
-  MVIT_EPI_SWIGLU = 4,     /* g = acc(B)+bias, u = acc(B2)+bias2; aux[m,n]=g, aux[m,aux_off+n]=u; C = silu(g)*u */
+  MVIT_EPI_SWIGLU = 4,     /* g = acc(B)+bias, u = acc(B2)+bias2; aux[m,n]=g, aux[m,aux_off+n]=u; C = silu(g)*u
+                              (aux may be null: a forward that will not be differentiated gets C alone)  */
   MVIT_EPI_SWIGLU_BWD = 5, /* dh = acc; (g,u) = R[m,n], R[m,aux_off+n]; C[m,n]=dg, C[m,aux_off+n]=du */
   MVIT_EPI_GELU_BWD = 6,   /* C = acc * gelu_erf'(R[m,n])                                     */
   MVIT_EPI_ACCUM = 7       /* C = C + acc                                                     */

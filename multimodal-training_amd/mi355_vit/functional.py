@@ -118,9 +118,15 @@ class AttnGeometry:
 
 
 def _block_forward(x: torch.Tensor, W: BlockWeights, geo: AttnGeometry, eps: float,
-                   attn_out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> Tuple[torch.Tensor, tuple]:
+                   attn_out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, *,
+                   for_backward: bool = True, output: bool = True) -> Tuple[Optional[torch.Tensor], tuple]:
     """``attn_out`` = (o, lse) kept from an earlier run of the same block on the same input: the attention product is
-    then not computed again (the recomputation of a checkpointed block)."""
+    then not computed again (the recomputation of a checkpointed block).
+
+    ``for_backward=False``: nothing but the block's output (and the attention output) will be used, so the gate / up
+    pre-activations are not written (the first run of a checkpointed block).  ``output=False``: the block's output is
+    not wanted, so the down projection is skipped (the re-run of a checkpointed block: the backward reads `h`, not
+    `x2`)."""
     S, C = x.shape
     H, hd = geo.nheads, geo.head_dim
     n1, rstd1 = ops.rmsnorm_fwd(x, W.norm1.view(-1), eps)
@@ -135,13 +141,15 @@ def _block_forward(x: torch.Tensor, W: BlockWeights, geo: AttnGeometry, eps: flo
     x1 = torch.empty_like(x)
     ops.gemm(o, W.wproj, x1, epilogue=E.EPI_BIAS_RES, bias=W.bproj.view(-1), residual=x)
     n2, rstd2 = ops.rmsnorm_fwd(x1, W.norm2.view(-1), eps)
-    gu = torch.empty(S, 2 * W.Ipad, dtype=x.dtype, device=x.device)
+    gu = torch.empty(S, 2 * W.Ipad, dtype=x.dtype, device=x.device) if for_backward else None
     h = torch.empty(S, W.Ipad, dtype=x.dtype, device=x.device)
     bgu = W.bgu.view(-1)
     ops.gemm(n2, W.wgu[: W.Ipad], h, epilogue=E.EPI_SWIGLU, b2=W.wgu[W.Ipad :], bias=bgu[: W.Ipad], bias2=bgu[W.Ipad :],
              aux=gu, aux_off=W.Ipad)
-    x2 = torch.empty_like(x)
-    ops.gemm(h, W.wdown, x2, epilogue=E.EPI_BIAS_RES, bias=W.bdown.view(-1), residual=x1)
+    x2 = None
+    if output:
+        x2 = torch.empty_like(x)
+        ops.gemm(h, W.wdown, x2, epilogue=E.EPI_BIAS_RES, bias=W.bdown.view(-1), residual=x1)
     return x2, (rstd1, n1, qkv, o, lse, x1, rstd2, n2, gu, h)
 
 
@@ -229,7 +237,10 @@ class VisionBlockFn(torch.autograd.Function):
     def forward(ctx, x, holder, geo: AttnGeometry, eps: float, checkpoint: bool, *params):
         W = holder.packed(x.dtype)
         x = x.contiguous()
-        x2, saved = _block_forward(x, W, geo, eps)
+        differentiated = any(ctx.needs_input_grad)  # False under torch.no_grad() and for frozen inputs and weights
+        x2, saved = _block_forward(x, W, geo, eps, for_backward=differentiated and not checkpoint)
+        if not differentiated:
+            return x2
         ctx.holder, ctx.geo, ctx.eps, ctx.checkpoint = holder, geo, eps, checkpoint
         ctx.gdt = {name: p.dtype for name, p in zip(BLOCK_PARAM_ORDER, params)}
         ctx.x = x
@@ -245,7 +256,7 @@ class VisionBlockFn(torch.autograd.Function):
         if saved is None:
             ops.recomputing = True
             try:
-                _, saved = _block_forward(x, W, geo, ctx.eps, ctx.attn_out)
+                _, saved = _block_forward(x, W, geo, ctx.eps, ctx.attn_out, output=False)
             finally:
                 ops.recomputing = False
         dx, grads = _block_backward(dx2, x, saved, W, geo, ctx.gdt)

@@ -344,6 +344,10 @@ def test_gemm_gelu_and_swiglu_epilogues(dtype):
     assert max_rel_err(gu[:, :I], gr) < TOL[dtype] and max_rel_err(gu[:, Ipad : Ipad + I], ur) < TOL[dtype]
     assert max_rel_err(h[:, :I], F.silu(gr) * ur) < TOL[dtype]
     assert (h[:, I:] == 0).all() and (gu[:, I:Ipad] == 0).all() and (gu[:, Ipad + I :] == 0).all()
+    # without aux (a forward that will not be differentiated): the same product, bit for bit, and nothing else written
+    h_only = torch.full((M, Ipad), float("nan"), dtype=dtype, device=DEV)
+    ops.gemm(a.to(DEV), wgu[:Ipad], h_only, epilogue=E.EPI_SWIGLU, b2=wgu[Ipad:], bias=bgu[:Ipad], bias2=bgu[Ipad:], aux_off=Ipad)
+    assert torch.equal(h_only.view(torch.uint8), h.view(torch.uint8))
     # backward epilogue: (dg, du) from dh = dx . Wdown, Wdown stored [C, Ipad] with zero padding columns
     Cc = 256
     dx, wd = _rand((M, Cc), dtype, 9), torch.zeros(Cc, Ipad, dtype=dtype)
