@@ -4,7 +4,7 @@ vision tower (bf16).  Default workload: one 3584 x 3584 image = 65,536 patches w
 checkpointing (the largest single-GPU configuration); the 8-image ragged batch (cfg2) and the video (cfg5) are
 timed beside it and reported under "other_workloads".
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg5|cfg1]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg5|cfg1|sample_yaml]
 
 One "step" = zero_grad, forward, backward with a fixed upstream gradient (the optimizer is not part of the
 path; "with_optimizer_step" reports the same loop with gradient norm, clipping and one Adam step added).  Inputs
@@ -54,6 +54,11 @@ def make_workload(name: str):
     if name == "cfg5":
         return ("full tower, video 16 frames 448x784 = 8x32x56 = 14,336 patches (seed 3)",
                 FULL_TOWER, torch.bfloat16, torch.tensor([[8, 32, 56]]), 3, False)
+    if name == "sample_yaml":
+        # the reference's own sample configuration (configs/sample.yaml:10,29,67-68): batch_size 4, min_pixels = max_pixels
+        # = 802,816 (896 x 896 px = 64 x 64 patches per image), bfloat16, activation checkpointing on
+        return ("full tower, 4 images 896x896 = 16,384 patches, per-block activation checkpointing (the reference's sample.yaml)",
+                FULL_TOWER, torch.bfloat16, torch.tensor([[1, 64, 64]] * 4), 4, True)
     if name == "cfg1":
         kw = dict(FULL_TOWER, depth=4, out_hidden_size=2048, fullatt_block_indexes=[3])
         return ("reduced tower depth 4, fp32, 2 images 224x224", kw, torch.float32, torch.tensor([[1, 16, 16], [1, 16, 16]]), 0, False)
@@ -537,7 +542,7 @@ def main() -> None:
     optimizer = handoff = input_side = with_opt = None
     others = None
     if not args.no_other_workloads and cfg_kw == FULL_TOWER:
-        others = {name: side_leg(other_workload, name) for name in ("cfg2", "cfg3", "cfg5") if name != args.workload}
+        others = {name: side_leg(other_workload, name) for name in ("cfg2", "cfg3", "cfg5", "sample_yaml") if name != args.workload}
         # the 65,536-patch image with every activation kept (no block is run twice): what 288 GB of HBM allow;
         # reported beside the metric, which stays on the configuration as it is named (checkpointing per block)
         others["cfg3_all_activations_kept"] = side_leg(other_workload, "cfg3", False)
