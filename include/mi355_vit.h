@@ -154,8 +154,10 @@ typedef struct mvit_gemm_args {
                       fp32 column sums of C per 256-row tile, [ceil(M/256)][ldc] (columns [0,N) and
                       [aux_off, aux_off+N) are written); add the rows with mvit_reduce_partials for the bias gradient */
   int64_t workspace_bytes;
-  int split_k;   /* <= 1: one work-group per tile walks all of K.  > 1 (EPI_NONE only): K is cut in split_k slices
-                    whose fp32 partial tiles go to `workspace` and are summed by a second kernel (fixed order) */
+  int split_k;   /* <= 1: one work-group per tile walks all of K.  > 1 (EPI_NONE, EPI_BIAS, EPI_BIAS_RES): K is cut in
+                    split_k slices whose fp32 partial tiles go to `workspace`; a second kernel sums them in a fixed
+                    order and applies the epilogue (few output tiles, long contraction: weight gradients, and every
+                    GEMM of a batch of a few hundred patches) */
 } mvit_gemm_args;
 
 /* C[M,N] = epilogue(sum_k A[m,k] * B[n,k]).  Operands must be 16-byte aligned with lda/ldb multiples of

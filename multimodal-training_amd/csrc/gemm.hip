@@ -36,6 +36,7 @@ struct GemmParams {
   void* aux;
   int64_t ldaux;
   int64_t aux_off;
+  int reduce_epi;  // split_k > 1: the epilogue that the reduction over the K slices applies (none, bias, bias + residual)
   int tiles_m, tiles_n;
   int split_k;        // K slices (1 = none)
   int64_t k_chunk;    // K extent of one slice (multiple of BK)
@@ -1240,11 +1241,13 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
   }
 }
 
-// C[m, n] = sum over slices of the fp32 partial tiles (fixed order, so the result is reproducible).
-// VEC: four consecutive columns per thread (N, ldc and the pointers allow 16-byte accesses).
-template <typename TO, bool VEC>
+// C[m, n] = epilogue(sum over slices of the fp32 partial tiles) (fixed order, so the result is reproducible); the
+// epilogue is none, + bias[n] or + bias[n] + R[m, n], in the order of the one-pass kernels' epilogue.
+// VEC: four consecutive columns per thread (N, the pitches and the pointers allow vector accesses).
+template <typename T, typename TO, bool VEC>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, int split_k, int64_t M, int64_t N,
-                                                            TO* __restrict__ C, int64_t ldc) {
+                                                            TO* __restrict__ C, int64_t ldc, int epi, const T* __restrict__ bias,
+                                                            const T* __restrict__ R, int64_t ldr) {
   const int64_t total = M * N;
   if constexpr (VEC) {
     const int64_t quads = total / 4, nq = N / 4;
@@ -1254,7 +1257,16 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
         const f32x4 v = *reinterpret_cast<const f32x4*>(ws + (int64_t)k * total + 4 * i);
         s = f32x4{s[0] + v[0], s[1] + v[1], s[2] + v[2], s[3] + v[3]};
       }
-      TO* c = C + (i / nq) * ldc + (i % nq) * 4;
+      const int64_t m = i / nq, n = (i % nq) * 4;
+      if (epi != MVIT_EPI_NONE) {
+        const auto b = *reinterpret_cast<const T __attribute__((ext_vector_type(4)))*>(bias + n);
+        s = f32x4{s[0] + to_f32(b[0]), s[1] + to_f32(b[1]), s[2] + to_f32(b[2]), s[3] + to_f32(b[3])};
+      }
+      if (epi == MVIT_EPI_BIAS_RES) {
+        const auto r = *reinterpret_cast<const T __attribute__((ext_vector_type(4)))*>(R + m * ldr + n);
+        s = f32x4{s[0] + to_f32(r[0]), s[1] + to_f32(r[1]), s[2] + to_f32(r[2]), s[3] + to_f32(r[3])};
+      }
+      TO* c = C + m * ldc + n;
       if constexpr (sizeof(TO) == 2) *reinterpret_cast<bf16x4*>(c) = bf16x4{(bf16_t)s[0], (bf16_t)s[1], (bf16_t)s[2], (bf16_t)s[3]};
       else *reinterpret_cast<f32x4*>(c) = s;
     }
@@ -1262,18 +1274,26 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
       float s = 0.f;
       for (int k = 0; k < split_k; ++k) s += ws[(int64_t)k * total + i];
-      C[(i / N) * ldc + (i % N)] = from_f32<TO>(s);
+      const int64_t m = i / N, n = i % N;
+      if (epi != MVIT_EPI_NONE) s += to_f32(bias[n]);
+      if (epi == MVIT_EPI_BIAS_RES) s += to_f32(R[m * ldr + n]);
+      C[m * ldc + n] = from_f32<TO>(s);
     }
   }
 }
-template <typename TO>
+template <typename T, typename TO>
 void launch_splitk_reduce(const GemmParams& p, hipStream_t stream) {
   const int64_t elems = p.M * p.N;
-  const bool vec = p.N % 4 == 0 && p.ldc % 4 == 0 && mvit_aligned16(p.workspace) && (reinterpret_cast<uintptr_t>(p.C) % (4 * sizeof(TO))) == 0;
+  const int epi = p.reduce_epi;
+  const T* bias = static_cast<const T*>(p.bias);
+  const T* R = static_cast<const T*>(p.R);
+  bool vec = p.N % 4 == 0 && p.ldc % 4 == 0 && mvit_aligned16(p.workspace) && (reinterpret_cast<uintptr_t>(p.C) % (4 * sizeof(TO))) == 0;
+  if (epi != MVIT_EPI_NONE) vec = vec && reinterpret_cast<uintptr_t>(bias) % (4 * sizeof(T)) == 0;
+  if (epi == MVIT_EPI_BIAS_RES) vec = vec && p.ldr % 4 == 0 && reinterpret_cast<uintptr_t>(R) % (4 * sizeof(T)) == 0;
   const int64_t items = vec ? elems / 4 : elems;
   const int rgrid = (int)((items + 255) / 256 < 8192 ? (items + 255) / 256 : 8192);
-  if (vec) hipLaunchKernelGGL((splitk_reduce_kernel<TO, true>), rgrid, 256, 0, stream, p.workspace, p.split_k, p.M, p.N, static_cast<TO*>(p.C), p.ldc);
-  else hipLaunchKernelGGL((splitk_reduce_kernel<TO, false>), rgrid, 256, 0, stream, p.workspace, p.split_k, p.M, p.N, static_cast<TO*>(p.C), p.ldc);
+  if (vec) hipLaunchKernelGGL((splitk_reduce_kernel<T, TO, true>), rgrid, 256, 0, stream, p.workspace, p.split_k, p.M, p.N, static_cast<TO*>(p.C), p.ldc, epi, bias, R, p.ldr);
+  else hipLaunchKernelGGL((splitk_reduce_kernel<T, TO, false>), rgrid, 256, 0, stream, p.workspace, p.split_k, p.M, p.N, static_cast<TO*>(p.C), p.ldc, epi, bias, R, p.ldr);
 }
 
 template <typename T, typename TO, bool TA, bool TB, int EPI, int VAR>
@@ -1298,7 +1318,7 @@ int launch(const GemmParams& p, hipStream_t stream) {
   hipLaunchKernelGGL(kern, grid, W::NTHREADS, lds, stream, p);
   MVIT_CHECK_LAUNCH("gemm");
   if (p.split_k > 1) {
-    launch_splitk_reduce<TO>(p, stream);
+    launch_splitk_reduce<T, TO>(p, stream);
     MVIT_CHECK_LAUNCH("gemm split-k reduce");
   }
   return MVIT_OK;
@@ -1333,7 +1353,7 @@ int launch_dl(const GemmParams& p, hipStream_t stream) {
   hipLaunchKernelGGL(kern, grid, D::NTHREADS, lds, stream, p);
   MVIT_CHECK_LAUNCH("gemm");
   if (p.split_k > 1) {
-    launch_splitk_reduce<TO>(p, stream);
+    launch_splitk_reduce<bf16_t, TO>(p, stream);
     MVIT_CHECK_LAUNCH("gemm split-k reduce");
   }
   return MVIT_OK;
@@ -1467,7 +1487,7 @@ extern "C" int mvit_patch_embed_frames(const mvit_image* images, int n_images, i
   MVIT_REQUIRE(tm * tn < (1ll << 30), "patch_embed_frames: too many tiles");
   p.tiles_m = (int)tm; p.tiles_n = (int)tn;
   p.panel_w = tn <= 6 ? (int)tn : 4;
-  p.split_k = 1; p.k_chunk = PX_K;
+  p.split_k = 1; p.k_chunk = PX_K; p.reduce_epi = MVIT_EPI_NONE;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (out_dtype == MVIT_BF16) return launch_dl<bf16_t, false, false, MVIT_EPI_NONE, 4, 8, false, true>(p, s);
   return launch_dl<float, false, false, MVIT_EPI_NONE, 4, 8, false, true>(p, s);
@@ -1488,7 +1508,7 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
   else MVIT_REQUIRE(a->lda >= (a->M + vec - 1) / vec * vec, "gemm: transposed A needs lda=%lld >= M=%lld rounded up to %d", (long long)a->lda, (long long)a->M, vec);
   if (!a->trans_b) MVIT_REQUIRE(a->K % vec == 0 && a->ldb >= a->K, "gemm: K=%lld must be a multiple of %d (ldb=%lld)", (long long)a->K, vec, (long long)a->ldb);
   else MVIT_REQUIRE(a->ldb >= (a->N + vec - 1) / vec * vec, "gemm: transposed B needs ldb=%lld >= N=%lld rounded up to %d", (long long)a->ldb, (long long)a->N, vec);
-  const int epi = a->epilogue;
+  int epi = a->epilogue;
   if (epi == MVIT_EPI_BIAS_RES || epi == MVIT_EPI_GELU_BWD || epi == MVIT_EPI_SWIGLU_BWD) MVIT_REQUIRE(a->R, "gemm: epilogue %d needs R", epi);
   if (epi == MVIT_EPI_BIAS_GELU) MVIT_REQUIRE(a->aux, "gemm: epilogue %d needs aux", epi);
   if (epi == MVIT_EPI_SWIGLU) MVIT_REQUIRE(a->B2 && !a->trans_a && !a->trans_b, "gemm: SWIGLU needs B2 and untransposed operands");
@@ -1509,7 +1529,7 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
   MVIT_REQUIRE(tm * tn < (1ll << 30), "gemm: too many tiles");
   p.tiles_m = (int)tm; p.tiles_n = (int)tn;
   p.panel_w = tn <= 6 ? (int)tn : 4;
-  p.split_k = 1; p.k_chunk = a->K; p.workspace = nullptr;
+  p.split_k = 1; p.k_chunk = a->K; p.workspace = nullptr; p.reduce_epi = MVIT_EPI_NONE;
   p.colsum = nullptr;
   if (epi == MVIT_EPI_SWIGLU_BWD && a->workspace) {
     MVIT_REQUIRE(mvit_aligned16(a->workspace) && a->workspace_bytes >= (int64_t)sizeof(float) * tm * a->ldc,
@@ -1520,11 +1540,18 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
     const int bk = a->dtype == MVIT_BF16 ? 64 : 16;
     const int64_t chunk = ((a->K + a->split_k - 1) / a->split_k + bk - 1) / bk * bk;
     const int64_t slices = (a->K + chunk - 1) / chunk;  // never an empty slice
-    MVIT_REQUIRE(epi == MVIT_EPI_NONE, "gemm: split_k is only available with EPI_NONE");
+    MVIT_REQUIRE(epi == MVIT_EPI_NONE || epi == MVIT_EPI_BIAS || epi == MVIT_EPI_BIAS_RES,
+                 "gemm: split_k is available with the plain, bias and bias + residual epilogues (got %d)", epi);
+    if (epi != MVIT_EPI_NONE) MVIT_REQUIRE(a->bias, "gemm: split_k with epilogue %d needs bias", epi);
     MVIT_REQUIRE(a->workspace && mvit_aligned16(a->workspace) && a->workspace_bytes >= (int64_t)sizeof(float) * slices * a->M * a->N,
                  "gemm: split_k=%d needs a 16-byte aligned workspace of %lld bytes", a->split_k, (long long)(sizeof(float) * slices * a->M * a->N));
     MVIT_REQUIRE(tm * tn * slices < (1ll << 30), "gemm: too many tiles");
-    if (slices > 1) { p.split_k = (int)slices; p.k_chunk = chunk; p.workspace = static_cast<float*>(a->workspace); }
+    if (slices > 1) {
+      // the main kernel leaves fp32 partial tiles; the reduction over the slices applies the epilogue
+      p.split_k = (int)slices; p.k_chunk = chunk; p.workspace = static_cast<float*>(a->workspace);
+      p.reduce_epi = epi;
+      epi = MVIT_EPI_NONE;
+    }
   }
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (a->dtype == MVIT_BF16) {

@@ -333,8 +333,8 @@ def gemm(
         args.aux, args.ldaux = aux.data_ptr(), aux.stride(0)
     args.aux_off = aux_off
     if split_k > 1:
-        if epilogue != _lib.EPI_NONE:
-            raise ValueError("gemm: split_k needs the plain epilogue")
+        if epilogue not in (_lib.EPI_NONE, _lib.EPI_BIAS, _lib.EPI_BIAS_RES):
+            raise ValueError("gemm: split_k needs the plain, the bias or the bias + residual epilogue")
         ws = torch.empty(split_k * M * N, dtype=torch.float32, device=a.device)
         args.workspace, args.workspace_bytes, args.split_k = ws.data_ptr(), ws.numel() * 4, split_k
     if colsum_partial is not None:
@@ -355,7 +355,9 @@ _N_CU = 256  # MI355X compute units; one 256x256 GEMM work-group runs per CU
 
 @functools.lru_cache(maxsize=None)
 def wgrad_split_k(out_rows: int, out_cols: int, k: int) -> int:
-    """K slices for a weight-gradient GEMM: few output tiles (256x256) but a long contraction (the tokens).
+    """K slices for a GEMM with few output tiles (256x256) and a long contraction: the weight gradients (contraction
+    over the tokens) at any batch size, and the forward / input-gradient GEMMs of a small batch (a few hundred to a few
+    thousand patches give 5 to 80 tiles for 256 compute units; from about 25,000 patches on the answer is 1).
 
     Picks the slice count with the lowest modelled time.  Work items (tiles x slices) run in rounds of one per
     CU, so the count should fill whole rounds; every slice costs an fp32 partial tile that a second kernel
@@ -376,6 +378,9 @@ def wgrad_split_k(out_rows: int, out_cols: int, k: int) -> int:
         if best_t is None or t < best_t:
             best, best_t = sk, t
     return best
+
+
+split_k_for = wgrad_split_k  # the same model, under the name the forward and input-gradient GEMMs call it by
 
 
 # ------------------------------------------------------------------------------ attention

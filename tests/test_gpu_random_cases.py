@@ -44,7 +44,7 @@ def _to_device_keeping_pitch(t):
 def test_gemm_random_shapes_layouts_and_epilogues(seed):
     """out = epilogue(op(A) op(B)^T) for random M, N, K (tile multiples, single rows, odd edges), the three operand
     layouts the library builds, padded row pitches on every operand and on the output, bias / bias + residual /
-    accumulate epilogues and K slices, against float32 matmul on the CPU; columns of the output buffer beyond N keep
+    accumulate epilogues and K slices (with the plain, bias and bias + residual epilogues), against float32 matmul on the CPU; columns of the output buffer beyond N keep
     their contents."""
     from mi355_vit import _lib as E
     from mi355_vit import ops
@@ -58,7 +58,7 @@ def test_gemm_random_shapes_layouts_and_epilogues(seed):
         ta, tb = rnd.choice([(False, False), (False, True), (True, True)])
         K = rnd.randint(1, 1200) if ta else vec * rnd.randint(1, 150)  # transposed operands: any contraction length
         epi = rnd.choice([E.EPI_NONE, E.EPI_NONE, E.EPI_BIAS, E.EPI_ACCUM] + ([] if tb else [E.EPI_BIAS_RES]))
-        split = rnd.choice([1, 1, 2, 3]) if epi == E.EPI_NONE and K >= 64 else 1
+        split = rnd.choice([1, 1, 2, 3]) if epi in (E.EPI_NONE, E.EPI_BIAS, E.EPI_BIAS_RES) and K >= 64 else 1
         out_dtype = dtype if dtype == torch.float32 else rnd.choice([torch.bfloat16, torch.float32])
         ldc = N + rnd.choice([0, 0, 3, 8])
         g = torch.Generator().manual_seed(1000 * seed + case)

@@ -367,3 +367,53 @@ def test_windowed_block_on_each_sequence_parallel_share_equals_the_unsharded_blo
     assert torch.equal(spu.gather_rank_packs(outs, lm), y_full.detach())
     assert torch.equal(spu.gather_rank_packs(dxs, lm), xf.grad)
     assert sum(o.shape[0] for o in outs) == S and min(o.shape[0] for o in outs) > 0
+
+
+def test_a_step_recorded_in_a_hip_graph_replays_bit_identically():
+    """The library's launches allocate nothing, wait for nothing and use no stream but the caller's (the eager backward's
+    second stream joins through events), so a whole forward and a whole backward can be recorded in HIP graphs.  Three
+    replays with different inputs, eager steps and synchronisations between them, each equal to the eager step bit for
+    bit (kernel order and arguments are the eager ones)."""
+    print("[case] forward and backward recorded in HIP graphs", flush=True)
+    kw = dict(depth=3, hidden_size=1280, intermediate_size=3420, num_heads=16, out_hidden_size=512, fullatt_block_indexes=[1])
+    model = _build(kw, 5, torch.bfloat16).to(DEV).train()
+    model.gradient_checkpointing_enable()
+    grid = torch.tensor([[1, 18, 22], [2, 8, 12], [1, 34, 16]])  # a host tensor: planning needs no device read-back
+    S = int(grid.prod(dim=1).sum())
+    params = list(model.parameters())
+
+    def inputs(seed):
+        g = torch.Generator().manual_seed(seed)
+        return torch.randn(S, 1176, generator=g).to(torch.bfloat16).to(DEV), torch.randn(S // 4, 512, generator=g).to(torch.bfloat16).to(DEV)
+
+    def eager(px, gout):
+        model.zero_grad(set_to_none=True)
+        out = model(hidden_states=px, grid_thw=grid)
+        out.backward(gout)
+        torch.cuda.synchronize()
+        return out.detach().clone(), [p.grad.detach().clone() for p in params]
+
+    static_px, static_gout = inputs(0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # plans, packed weights and library handles come into being before the recording
+        for _ in range(2):
+            torch.autograd.grad(model(hidden_states=static_px, grid_thw=grid), params, static_gout)
+    torch.cuda.current_stream().wait_stream(side)
+    pool = torch.cuda.graph_pool_handle()
+    fwd, bwd = torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()
+    with torch.cuda.graph(fwd, pool=pool):
+        static_out = model(hidden_states=static_px, grid_thw=grid)
+    with torch.cuda.graph(bwd, pool=pool):
+        static_grads = torch.autograd.grad(static_out, params, static_gout)
+    for seed in (1, 2, 1):
+        px, gout = inputs(seed)
+        out_e, grads_e = eager(px, gout)
+        static_px.copy_(px)
+        static_gout.copy_(gout)
+        fwd.replay()
+        bwd.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_out.detach(), out_e), f"output, inputs {seed}"
+        for i, (a, b) in enumerate(zip(static_grads, grads_e)):
+            assert torch.equal(a, b), f"gradient {i}, inputs {seed}"
