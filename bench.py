@@ -4,7 +4,7 @@ vision tower (bf16).  Default workload: one 3584 x 3584 image = 65,536 patches w
 checkpointing (the largest single-GPU configuration); the 8-image ragged batch (cfg2) and the video (cfg5) are
 timed beside it and reported under "other_workloads".
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg5|cfg1|sample_yaml]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg5|cfg1|sample_yaml|one_224]
 
 One "step" = zero_grad, forward, backward with a fixed upstream gradient (the optimizer is not part of the
 path; "with_optimizer_step" reports the same loop with gradient norm, clipping and one Adam step added).  Inputs
@@ -59,6 +59,9 @@ def make_workload(name: str):
         # = 802,816 (896 x 896 px = 64 x 64 patches per image), bfloat16, activation checkpointing on
         return ("full tower, 4 images 896x896 = 16,384 patches, per-block activation checkpointing (the reference's sample.yaml)",
                 FULL_TOWER, torch.bfloat16, torch.tensor([[1, 64, 64]] * 4), 4, True)
+    if name == "one_224":
+        return ("full tower, one 224x224 image = 256 patches (a batch too small to fill the GPU: what a step costs at least)",
+                FULL_TOWER, torch.bfloat16, torch.tensor([[1, 16, 16]]), 5, False)
     if name == "cfg1":
         kw = dict(FULL_TOWER, depth=4, out_hidden_size=2048, fullatt_block_indexes=[3])
         return ("reduced tower depth 4, fp32, 2 images 224x224", kw, torch.float32, torch.tensor([[1, 16, 16], [1, 16, 16]]), 0, False)
