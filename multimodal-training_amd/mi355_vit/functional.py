@@ -166,7 +166,8 @@ def _block_backward(dx2: torch.Tensor, x: torch.Tensor, saved: tuple, W: BlockWe
 
     def off_chain(fn):
         # work that feeds nothing else in this block (weight and bias gradients) runs on the second stream, after
-        # the point its inputs are complete on the main stream, and is joined before the gradients are handed back
+        # the point its inputs are complete on the main stream, and is joined before the gradients are handed back;
+        # one event and one stream switch per point serve the bias and the weight gradient that start there
         if side is None:
             return fn()
         ev = torch.cuda.Event()
@@ -176,37 +177,32 @@ def _block_backward(dx2: torch.Tensor, x: torch.Tensor, saved: tuple, W: BlockWe
             return fn()
 
     def wgrad(dy, act, out, **kw):
-        split = ops.wgrad_split_k(out.shape[0], out.shape[1], S)
-        off_chain(lambda: ops.gemm(dy, act, out, trans_a=True, trans_b=True, split_k=split, **kw))
+        ops.gemm(dy, act, out, trans_a=True, trans_b=True, split_k=ops.wgrad_split_k(out.shape[0], out.shape[1], S), **kw)
 
     # ---- MLP: x2 = x1 + down(silu(g) * u)
-    g_bd = off_chain(lambda: ops.colsum(dx2, gdt["mlp.down_proj.bias"]))
     g_wd = torch.empty(C, I, dtype=gdt["mlp.down_proj.weight"], device=dev)
-    wgrad(dx2, h, g_wd, n=I)
+    g_bd = off_chain(lambda: (ops.colsum(dx2, gdt["mlp.down_proj.bias"]), wgrad(dx2, h, g_wd, n=I))[0])
     dgu = torch.empty(S, 2 * Ipad, dtype=x.dtype, device=dev)
     # the epilogue also hands back per-tile column sums of dgu: the gate / up bias gradient without re-reading dgu
     part = torch.empty(-(-S // 256), 2 * Ipad, dtype=torch.float32, device=dev)
     ops.gemm(dx2, W.wdown, dgu, trans_b=True, epilogue=E.EPI_SWIGLU_BWD, residual=gu, aux_off=Ipad, colsum_partial=part)
-    g_bgu = off_chain(lambda: ops.reduce_partials(part, gdt["mlp.gate_proj.bias"]))
     g_wgu = torch.empty(2 * Ipad, C, dtype=gdt["mlp.gate_proj.weight"], device=dev)
-    wgrad(dgu, n2, g_wgu)
+    g_bgu = off_chain(lambda: (ops.reduce_partials(part, gdt["mlp.gate_proj.bias"]), wgrad(dgu, n2, g_wgu))[0])
     dn2 = torch.empty_like(x)
     ops.gemm(dgu, W.wgu, dn2, trans_b=True)
     dx1, g_n2 = ops.rmsnorm_bwd(dn2, x1, W.norm2.view(-1), rstd2, dx_add=dx2, w_grad_dtype=gdt["norm2.weight"])
 
     # ---- attention: x1 = x + proj(attn(rope(qkv(norm1(x)))))
-    g_bp = off_chain(lambda: ops.colsum(dx1, gdt["attn.proj.bias"]))
     g_wp = torch.empty(C, C, dtype=gdt["attn.proj.weight"], device=dev)
-    wgrad(dx1, o, g_wp)
+    g_bp = off_chain(lambda: (ops.colsum(dx1, gdt["attn.proj.bias"]), wgrad(dx1, o, g_wp))[0])
     d_o = dn2  # reuse the buffer
     ops.gemm(dx1, W.wproj, d_o, trans_b=True)
     dqkv = torch.empty_like(qkv)
     ops.attn_bwd(qkv[:, :C], qkv[:, C : 2 * C], qkv[:, 2 * C :], o, d_o, lse, geo.cu, geo.max_seqlen, H, hd, hd**-0.5,
                  dqkv[:, :C], dqkv[:, C : 2 * C], dqkv[:, 2 * C :], seg_order=geo.order)
     ops.rope_(dqkv, geo.cos, geo.sin, 2 * H, hd, backward=True)
-    g_bqkv = off_chain(lambda: ops.colsum(dqkv, gdt["attn.q_proj.bias"]))
     g_wqkv = torch.empty(3 * C, C, dtype=gdt["attn.q_proj.weight"], device=dev)
-    wgrad(dqkv, n1, g_wqkv)
+    g_bqkv = off_chain(lambda: (ops.colsum(dqkv, gdt["attn.q_proj.bias"]), wgrad(dqkv, n1, g_wqkv))[0])
     dn1 = d_o
     ops.gemm(dqkv, W.wqkv, dn1, trans_b=True)
     dx, g_n1 = ops.rmsnorm_bwd(dn1, x, W.norm1.view(-1), rstd1, dx_add=dx1, w_grad_dtype=gdt["norm1.weight"])

@@ -60,10 +60,14 @@ def dt(t: torch.Tensor) -> int:
         raise TypeError(f"unsupported dtype {t.dtype} (float32 and bfloat16 only)") from None
 
 
+_current_raw_stream = torch._C._cuda_getCurrentRawStream  # the handle alone, without building a Stream object per launch
+
+
 def _stream(t: torch.Tensor) -> int:
     if not t.is_cuda:
         raise RuntimeError("mi355_vit kernels need tensors on the GPU; there is no CPU path")
-    return torch.cuda.current_stream(t.device).cuda_stream
+    index = t.device.index
+    return _current_raw_stream(torch.cuda.current_device() if index is None else index)
 
 
 def _p(t: Optional[torch.Tensor]) -> Optional[int]:

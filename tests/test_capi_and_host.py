@@ -178,3 +178,20 @@ def test_segment_lists_are_validated_on_the_host():
         except ValueError:
             continue
         raise AssertionError(f"accepted {cu}, total {total}, max {mx}, order {order}")
+
+
+def test_block_parameter_list_follows_the_declared_order():
+    """The block hands its 16 parameters to the kernels as a list built from the module dictionaries (no name lookups on
+    the hot path): it must be the parameters BLOCK_PARAM_ORDER names, in that order, also after one was replaced."""
+    import torch
+    from mi355_vit.config import Qwen2_5_VLVisionConfig
+    from mi355_vit.functional import BLOCK_PARAM_ORDER
+    from mi355_vit.modeling import Qwen2_5_VisionTransformerPretrainedModel
+
+    model = Qwen2_5_VisionTransformerPretrainedModel(Qwen2_5_VLVisionConfig(
+        depth=2, hidden_size=64, intermediate_size=100, num_heads=2, out_hidden_size=32, fullatt_block_indexes=[1]))
+    for blk in model.blocks:
+        assert all(p is blk.get_parameter(n) for p, n in zip(blk._block_params(), BLOCK_PARAM_ORDER, strict=True))
+    blk = model.blocks[0]
+    blk.attn.proj.weight = torch.nn.Parameter(torch.zeros(64, 64))
+    assert blk._block_params()[BLOCK_PARAM_ORDER.index("attn.proj.weight")] is blk.attn.proj.weight
