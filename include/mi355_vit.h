@@ -87,6 +87,14 @@ int mvit_reduce_partials(const float* partial, int n_partial, int64_t cols, void
 int mvit_rope(void* x, const float* cos, const float* sin, int64_t rows, int nheads, int head_dim,
               int64_t row_stride, int backward, int dtype, mvit_stream_t stream);
 
+/* mvit_rope with the first `lead_heads` heads also multiplied by `lead_scale` before the single rounding to the storage
+ * type (backward: after the transposed rotation).  The block passes its queries' softmax scale here
+ * (head_dim^-1/2 * log2 e, the factor `q * scaling` of modeling:298-321 / the softmax_scale of the flash-attention call
+ * :431-448 would apply) and calls the attention entry points with scale = 1 / log2 e: the scores then come from
+ * once-rounded operands, as the reference's do. */
+int mvit_rope_scaled(void* x, const float* cos, const float* sin, int64_t rows, int nheads, int head_dim,
+                     int64_t row_stride, int backward, int lead_heads, float lead_scale, int dtype, mvit_stream_t stream);
+
 /* dst[i, :] = src[index[i], :] for rows of row_bytes bytes (multiple of 2).  Bit-exact.
  * Replaces the window reorder x.view(M,4,C)[window_index] and its inverse, modeling:934-940, :1067-1068. */
 int mvit_gather_rows(const void* src, const int64_t* index, void* dst, int64_t n_rows, int64_t row_bytes,

@@ -229,10 +229,13 @@ __global__ __launch_bounds__(256) void colsum_kernel(const T* __restrict__ x, in
 // ------------------------------------------------------------------------------------------------
 // Rotary embedding in place.  A thread owns V consecutive elements of the first half of one head and
 // the matching V of the second half.  Algorithmic bytes per (row, head): 2*head_dim*e + table share.
+// The first `lead_heads` heads are multiplied by `lead_scale` before the one rounding to the storage type (the
+// queries of an attention layer take the softmax scale here, so that no later pass rounds them a second time).
 template <typename T, int V>
 __global__ __launch_bounds__(256) void rope_kernel(T* __restrict__ x, const float* __restrict__ cosb,
                                                    const float* __restrict__ sinb, int64_t rows, int nheads,
-                                                   int head_dim, int64_t row_stride, int backward) {
+                                                   int head_dim, int64_t row_stride, int backward, int lead_heads,
+                                                   float lead_scale) {
   typedef T vec_t __attribute__((ext_vector_type(V)));
   const int half = head_dim / 2;
   const int chunks = half / V;  // per head
@@ -243,6 +246,7 @@ __global__ __launch_bounds__(256) void rope_kernel(T* __restrict__ x, const floa
     const int h = (int)(rh % nheads);
     const int64_t r = rh / nheads;
     T* p = x + r * row_stride + (int64_t)h * head_dim + ch * V;
+    const float gain = h < lead_heads ? lead_scale : 1.f;
     const float* c = cosb + r * head_dim + ch * V;
     const float* s = sinb + r * head_dim + ch * V;
     vec_t lo, hi, olo, ohi;
@@ -265,8 +269,8 @@ __global__ __launch_bounds__(256) void rope_kernel(T* __restrict__ x, const floa
         oa = a * c0 + b * s1;
         ob = b * c1 - a * s0;
       }
-      olo[j] = from_f32<T>(oa);
-      ohi[j] = from_f32<T>(ob);
+      olo[j] = from_f32<T>(oa * gain);
+      ohi[j] = from_f32<T>(ob * gain);
     }
     if (V > 1) {
       *reinterpret_cast<vec_t*>(p) = olo;
@@ -491,6 +495,12 @@ int mvit_colsum(const void* x, int64_t ld, int64_t rows, int64_t cols, float* pa
 
 int mvit_rope(void* x, const float* cosb, const float* sinb, int64_t rows, int nheads, int head_dim, int64_t row_stride,
               int backward, int dtype, mvit_stream_t stream) {
+  return mvit_rope_scaled(x, cosb, sinb, rows, nheads, head_dim, row_stride, backward, 0, 1.f, dtype, stream);
+}
+
+int mvit_rope_scaled(void* x, const float* cosb, const float* sinb, int64_t rows, int nheads, int head_dim, int64_t row_stride,
+                     int backward, int lead_heads, float lead_scale, int dtype, mvit_stream_t stream) {
+  MVIT_REQUIRE(lead_heads >= 0 && lead_heads <= nheads, "rope: lead_heads=%d of %d heads", lead_heads, nheads);
   MVIT_REQUIRE(rows >= 0 && nheads > 0 && head_dim > 0 && head_dim % 2 == 0 && row_stride >= (int64_t)nheads * head_dim,
                "rope: bad shape rows=%lld heads=%d head_dim=%d stride=%lld", (long long)rows, nheads, head_dim, (long long)row_stride);
   if (rows == 0) return MVIT_OK;
@@ -500,18 +510,18 @@ int mvit_rope(void* x, const float* cosb, const float* sinb, int64_t rows, int n
   if (dtype == MVIT_BF16) {
     if (half % 8 == 0 && row_stride % 8 == 0 && mvit_aligned16(x)) {
       const int grid = clamp_grid((work_scalar / 8 + 255) / 256, 65535 * 16);
-      hipLaunchKernelGGL((rope_kernel<bf16_t, 8>), grid, 256, 0, S_(stream), (bf16_t*)x, cosb, sinb, rows, nheads, head_dim, row_stride, backward);
+      hipLaunchKernelGGL((rope_kernel<bf16_t, 8>), grid, 256, 0, S_(stream), (bf16_t*)x, cosb, sinb, rows, nheads, head_dim, row_stride, backward, lead_heads, lead_scale);
     } else {
       const int grid = clamp_grid((work_scalar + 255) / 256, 65535 * 16);
-      hipLaunchKernelGGL((rope_kernel<bf16_t, 1>), grid, 256, 0, S_(stream), (bf16_t*)x, cosb, sinb, rows, nheads, head_dim, row_stride, backward);
+      hipLaunchKernelGGL((rope_kernel<bf16_t, 1>), grid, 256, 0, S_(stream), (bf16_t*)x, cosb, sinb, rows, nheads, head_dim, row_stride, backward, lead_heads, lead_scale);
     }
   } else if (dtype == MVIT_F32) {
     if (half % 4 == 0 && row_stride % 4 == 0 && mvit_aligned16(x)) {
       const int grid = clamp_grid((work_scalar / 4 + 255) / 256, 65535 * 16);
-      hipLaunchKernelGGL((rope_kernel<float, 4>), grid, 256, 0, S_(stream), (float*)x, cosb, sinb, rows, nheads, head_dim, row_stride, backward);
+      hipLaunchKernelGGL((rope_kernel<float, 4>), grid, 256, 0, S_(stream), (float*)x, cosb, sinb, rows, nheads, head_dim, row_stride, backward, lead_heads, lead_scale);
     } else {
       const int grid = clamp_grid((work_scalar + 255) / 256, 65535 * 16);
-      hipLaunchKernelGGL((rope_kernel<float, 1>), grid, 256, 0, S_(stream), (float*)x, cosb, sinb, rows, nheads, head_dim, row_stride, backward);
+      hipLaunchKernelGGL((rope_kernel<float, 1>), grid, 256, 0, S_(stream), (float*)x, cosb, sinb, rows, nheads, head_dim, row_stride, backward, lead_heads, lead_scale);
     }
   } else {
     return mvit_set_error(MVIT_ERR_UNSUPPORTED, "rope: dtype %d", dtype);

@@ -66,6 +66,7 @@ PROTOTYPES = {
     "mvit_reduce_partials": [_vp, _i32, _i64, _vp, _i32, _vp],
     "mvit_colsum": [_vp, _i64, _i64, _i64, _vp, _i32, _i32, _vp],
     "mvit_rope": [_vp, _vp, _vp, _i64, _i32, _i32, _i64, _i32, _i32, _vp],
+    "mvit_rope_scaled": [_vp, _vp, _vp, _i64, _i32, _i32, _i64, _i32, _i32, C.c_float, _i32, _vp],
     "mvit_gather_rows": [_vp, _vp, _vp, _i64, _i64, _vp],
     "mvit_segment_copy": [_vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "mvit_pad_pack": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, C.c_uint32, _vp],

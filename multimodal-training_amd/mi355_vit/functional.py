@@ -50,6 +50,8 @@ class BlockWeights:
 
 
 # order of the parameter tensors handed to VisionBlockFn
+LOG2E = 1.4426950408889634  # log2(e): the attention kernels work in base-2 exponentials
+
 BLOCK_PARAM_ORDER = (
     "norm1.weight", "norm2.weight",
     "attn.q_proj.weight", "attn.q_proj.bias", "attn.k_proj.weight", "attn.k_proj.bias",
@@ -132,9 +134,13 @@ def _block_forward(x: torch.Tensor, W: BlockWeights, geo: AttnGeometry, eps: flo
     n1, rstd1 = ops.rmsnorm_fwd(x, W.norm1.view(-1), eps)
     qkv = torch.empty(S, 3 * C, dtype=x.dtype, device=x.device)
     ops.gemm(n1, W.wqkv, qkv, epilogue=E.EPI_BIAS, bias=W.bqkv.view(-1))
-    ops.rope_(qkv, geo.cos, geo.sin, 2 * H, hd)  # q and k are the first 2*H heads of every row
+    # q and k are the first 2*H heads of every row.  The queries leave the rotary pass multiplied by the softmax scale
+    # in base-2 units (Q_SCALE), in the same fp32 -> storage rounding as the rotation; the attention kernels then get
+    # scale = 1 / log2(e), for which their own pre-scaling of the queries is the identity.  Scores are computed from
+    # operands rounded once, as in the reference (the kernels alone would round q * scale a second time).
+    ops.rope_(qkv, geo.cos, geo.sin, 2 * H, hd, lead_heads=H, lead_scale=hd**-0.5 * LOG2E)
     if attn_out is None:
-        o, lse = ops.attn_fwd(qkv[:, :C], qkv[:, C : 2 * C], qkv[:, 2 * C :], geo.cu, geo.max_seqlen, H, hd, hd**-0.5,
+        o, lse = ops.attn_fwd(qkv[:, :C], qkv[:, C : 2 * C], qkv[:, 2 * C :], geo.cu, geo.max_seqlen, H, hd, 1.0 / LOG2E,
                               seg_order=geo.order)
     else:
         o, lse = attn_out
@@ -198,9 +204,10 @@ def _block_backward(dx2: torch.Tensor, x: torch.Tensor, saved: tuple, W: BlockWe
     d_o = dn2  # reuse the buffer
     ops.gemm(dx1, W.wproj, d_o, trans_b=True)
     dqkv = torch.empty_like(qkv)
-    ops.attn_bwd(qkv[:, :C], qkv[:, C : 2 * C], qkv[:, 2 * C :], o, d_o, lse, geo.cu, geo.max_seqlen, H, hd, hd**-0.5,
+    ops.attn_bwd(qkv[:, :C], qkv[:, C : 2 * C], qkv[:, 2 * C :], o, d_o, lse, geo.cu, geo.max_seqlen, H, hd, 1.0 / LOG2E,
                  dqkv[:, :C], dqkv[:, C : 2 * C], dqkv[:, 2 * C :], seg_order=geo.order)
-    ops.rope_(dqkv, geo.cos, geo.sin, 2 * H, hd, backward=True)
+    # dq arrives as the gradient with respect to the scaled, rotated queries: the same factor on the way back
+    ops.rope_(dqkv, geo.cos, geo.sin, 2 * H, hd, backward=True, lead_heads=H, lead_scale=hd**-0.5 * LOG2E)
     g_wqkv = torch.empty(3 * C, C, dtype=gdt["attn.q_proj.weight"], device=dev)
     g_bqkv = off_chain(lambda: (ops.colsum(dqkv, gdt["attn.q_proj.bias"]), wgrad(dqkv, n1, g_wqkv))[0])
     dn1 = d_o

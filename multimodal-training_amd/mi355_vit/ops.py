@@ -185,8 +185,10 @@ def colsum(x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
     return out
 
 
-def rope_(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, nheads: int, head_dim: int, backward: bool = False) -> torch.Tensor:
-    """In-place rotary embedding on the first nheads*head_dim columns of each row of x ([rows, >=nheads*head_dim])."""
+def rope_(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, nheads: int, head_dim: int, backward: bool = False,
+          lead_heads: int = 0, lead_scale: float = 1.0) -> torch.Tensor:
+    """In-place rotary embedding on the first nheads*head_dim columns of each row of x ([rows, >=nheads*head_dim]).
+    The first ``lead_heads`` heads are also multiplied by ``lead_scale`` before the one rounding to x's dtype."""
     _rowmajor(x, "rope x")
     rows = x.shape[0]
     for t in (cos, sin):
@@ -194,10 +196,13 @@ def rope_(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, nheads: int, he
             raise ValueError(f"rope: cos/sin must be contiguous fp32 [{rows}, {head_dim}]")
     if x.shape[1] < nheads * head_dim:
         raise ValueError("rope: row narrower than nheads*head_dim")
+    if not 0 <= lead_heads <= nheads:
+        raise ValueError(f"rope: lead_heads {lead_heads} of {nheads} heads")
     st = _stream(x)
     rc = _launch("rope", {"rows": rows, "nheads": nheads, "head_dim": head_dim, "esize": x.element_size()},
-                 lambda: _lib.load().mvit_rope(x.data_ptr(), cos.data_ptr(), sin.data_ptr(), rows, nheads, head_dim, x.stride(0), int(backward), dt(x), st))
-    _lib.check(rc, "mvit_rope")
+                 lambda: _lib.load().mvit_rope_scaled(x.data_ptr(), cos.data_ptr(), sin.data_ptr(), rows, nheads, head_dim, x.stride(0),
+                                                      int(backward), lead_heads, lead_scale, dt(x), st))
+    _lib.check(rc, "mvit_rope_scaled")
     return x
 
 

@@ -91,6 +91,58 @@ def test_rope_fwd_bwd(dtype, S, H, d):
     assert max_rel_err(gg, xin.grad.reshape(S, H * d)) < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_with_scaled_leading_heads(dtype):
+    """The first `lead_heads` heads leave the rotary pass multiplied by `lead_scale`, in the same rounding: bit-equal to
+    the oracle's rotation times the factor rounded once; the other heads and the columns behind them as without it."""
+    _announce(f"rope with scaled leading heads {dtype}")
+    ops = _ops()
+    S, H, d, lead, gain = 300, 6, 80, 3, 0.1613
+    x = _rand((S, H * d + 16), dtype, 0)
+    ang = torch.cat([_rand((S, d // 2), torch.float32, 1, 3.0)] * 2, dim=-1)
+    cos, sin = ang.cos(), ang.sin()
+    for backward in (False, True):
+        got = x.to(DEV).clone()
+        ops.rope_(got, cos.to(DEV), sin.to(DEV), H, d, backward=backward, lead_heads=lead, lead_scale=gain)
+        plain = x.to(DEV).clone()
+        ops.rope_(plain, cos.to(DEV), sin.to(DEV), H, d, backward=backward)
+        assert torch.equal(got[:, lead * d :], plain[:, lead * d :])
+        xin = x[:, : H * d].float().reshape(S, H, d).requires_grad_(backward)
+        if backward:
+            vit_oracle.rope_apply(xin, cos, sin).backward(x[:, : H * d].float().reshape(S, H, d))
+            rot = xin.grad
+        else:
+            rot = vit_oracle.rope_apply(xin, cos, sin)
+        want = (rot[:, :lead] * torch.tensor(gain, dtype=torch.float32)).reshape(S, lead * d)
+        assert max_rel_err(got[:, : lead * d], want) < (1e-6 if dtype == torch.float32 else 2.0**-8)
+
+
+def test_queries_scaled_in_the_rotary_pass_are_rounded_once():
+    """What the block does (queries take head_dim^-1/2 * log2 e in the rotary pass, attention called with scale
+    1 / log2 e) against handing bf16 queries to the attention entry point with the plain scale (which rounds q * scale
+    to bf16 a second time): with scores of standard deviation 9 the output error against float64 attention on the
+    unrounded queries falls from 2.5e-2 to 1.5e-2, the level of exact attention on queries rounded once."""
+    _announce("attention: queries scaled in the rotary pass")
+    ops = _ops()
+    S, H, d, LOG2E = 2048, 4, 80, 1.4426950408889634
+    g = torch.Generator().manual_seed(0)
+    q32 = torch.randn(S, H * d, generator=g) * 3.0  # fp32 queries as they leave the rotation, before any rounding
+    k = (torch.randn(S, H * d, generator=g) * 3.0).to(torch.bfloat16)
+    v = torch.randn(S, H * d, generator=g).to(torch.bfloat16)
+    cu = torch.tensor([0, S], dtype=torch.int32, device=DEV)
+    heads = lambda t: t.double().to(DEV).reshape(S, H, d).transpose(0, 1)  # noqa: E731
+    ref = (torch.softmax(heads(q32) @ heads(k).transpose(1, 2) * d**-0.5, -1) @ heads(v)).transpose(0, 1).reshape(S, H * d)
+    err = lambda o: float((o.double() - ref).abs().max() / ref.abs().max())  # noqa: E731
+    twice, _ = ops.attn_fwd(q32.to(torch.bfloat16).to(DEV), k.to(DEV), v.to(DEV), cu, S, H, d, d**-0.5)
+    once, _ = ops.attn_fwd((q32 * (d**-0.5 * LOG2E)).to(torch.bfloat16).to(DEV), k.to(DEV), v.to(DEV), cu, S, H, d, 1.0 / LOG2E)
+    # float64 attention on queries rounded to bf16 once, everything else exact: what no bf16 pipeline can beat by much
+    floor = err((torch.softmax(heads(q32.to(torch.bfloat16)) @ heads(k).transpose(1, 2) * d**-0.5, -1) @ heads(v)).transpose(0, 1).reshape(S, H * d))
+    e_twice, e_once = err(twice), err(once)
+    print(f"    output error: q rounded, then q * scale rounded {e_twice:.2e}; q * scale rounded once {e_once:.2e}; "
+          f"exact attention on once-rounded q {floor:.2e}", flush=True)
+    assert e_once < 2e-2 and e_once < 0.75 * e_twice and e_once < 1.5 * floor
+
+
 # ------------------------------------------------------------------------------------------ copies
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gather_rows_window_permutation_bit_exact(dtype):
