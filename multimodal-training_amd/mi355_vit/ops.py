@@ -60,7 +60,9 @@ def dt(t: torch.Tensor) -> int:
         raise TypeError(f"unsupported dtype {t.dtype} (float32 and bfloat16 only)") from None
 
 
-_current_raw_stream = torch._C._cuda_getCurrentRawStream  # the handle alone, without building a Stream object per launch
+# the current stream's handle alone, without building a Stream object per launch (a torch build without the direct
+# accessor goes through the object)
+_current_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None) or (lambda index: torch.cuda.current_stream(index).cuda_stream)
 
 
 def _stream(t: torch.Tensor) -> int:
