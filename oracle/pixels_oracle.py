@@ -7,9 +7,10 @@ The reference does not hold this code: ``python/data/preprocessing.py:134`` call
 ``transformers`` (pinned ``transformers==4.57.0`` in the reference's requirements.txt;
 ``models/qwen2_vl/image_processing_qwen2_vl.py``, ``Qwen2VLImageProcessor._preprocess``),
 and ``python/data/collator.py:134-156`` concatenates the per-sample results along dim 0.
-That library is not importable in this environment (the installed transformers needs
-torchvision for this module), so its published algorithm is restated here, for frames that
-are already resized (height and width multiples of patch * merge = 28):
+Version 4.57.0 is not installed; the installed transformers 5.15.0 holds the same processor with a PIL
+backend (``models/qwen2_vl/image_processing_pil_qwen2_vl.py``, ``Qwen2VLImageProcessorPil``), and the
+restatement below is held to it bit for bit.  The algorithm, for frames that are already resized
+(height and width multiples of patch * merge = 28):
 
   1. rescale: ``image.astype(float64) * (1 / 255)`` cast to float32   (image_transforms.rescale)
   2. normalise: ``(image - mean) / std`` in float32, mean / std = OPENAI_CLIP  (image_transforms.normalize)
@@ -31,8 +32,15 @@ column order         ``rows @ W.view(1280, 1176).T`` equals ``torch.nn.functiona
                      (2, 14, 14): the patch embedding the reference applies to it
                      (Qwen2_5_VisionPatchEmbed: Conv3d on rows viewed as
                      [-1, 3, 2, 14, 14])
-rescale / normalise  closed form in float64, agreement to 1 float32 ulp; exactness
-                     against the library itself: PARITY UNPINNED (library absent)
+rescale / normalise  closed form in float64, agreement to 1 float32 ulp
+the whole chain      ``smart_resize`` -> bicubic resize (oracle/resize_oracle.py) -> these rows
+                     equal ``Qwen2VLImageProcessorPil()(images=...)`` of transformers 5.15.0
+                     bit for bit (SHA-256 of the float32 ``pixel_values`` and sampled rows)
+                     on eight seeded images: no resize, rounding to multiples of 28,
+                     a 2000 x 3000 down-scale, the min-pixels clamp, a thin up-scale,
+                     custom pixel limits; vectors in tests/golden/processor_vectors.npz,
+                     written by tests/golden/make_processor_vectors.py.  Against 4.57.0
+                     itself (the reference's pin): not checked, that version is absent
 frame fill-up        still image: both temporal halves of a row equal; odd videos:
                      last row group uses the last frame twice
 ===================  ==============================================================

@@ -14,8 +14,9 @@ What it restates
 
 Pins (tests/test_oracle_resize.py): ``pil_resize`` is compared bit for bit with Pillow itself (the library is installed;
 pinned version of the reference: pillow 11.3.0, same algorithm) on random images over up- and down-scaling ratios,
-both filters, sizes down to 1 pixel; ``smart_resize`` against its three defining properties, hand-computed cases and
-an exhaustive scan for the rounding branch.
+both filters, sizes down to 1 pixel; ``smart_resize`` against its three defining properties, hand-computed cases, an
+exhaustive scan for the rounding branch, and 400 size / limit combinations tabulated from the library's own
+``smart_resize`` (transformers 5.15.0, tests/golden/processor_vectors.npz; tests/test_oracle_pixels.py).
 """
 
 from __future__ import annotations

@@ -1,6 +1,7 @@
-"""Pins oracle/pixels_oracle.py (decoded frames -> pixel_values rows) without the image-processor library, which is
-not importable here: row order against the position ids the model computes for each row, column order against
-Conv3d (the patch embedding the model applies), the arithmetic against its closed form, and the frame fill-up."""
+"""Pins oracle/pixels_oracle.py (decoded frames -> pixel_values rows): row order against the position ids the model
+computes for each row, column order against Conv3d (the patch embedding the model applies), the arithmetic against its
+closed form, the frame fill-up, and the whole chain (target size, bicubic resize, rescale, normalise, patch rows)
+against vectors written from the image-processor library itself (second half of this file)."""
 
 import numpy as np
 import pytest
@@ -97,3 +98,83 @@ def test_host_mirror_grid_and_guards_without_a_gpu():
             pixels.grid_thw_of([bad])
     with pytest.raises(RuntimeError, match="no CPU path"):
         pixels.patchify(frames[:1])
+
+
+# ---- the oracle against the image processor library itself ------------------------------------------------------
+# tests/golden/processor_vectors.npz is written by tests/golden/make_processor_vectors.py from
+# transformers.models.qwen2_vl.image_processing_pil_qwen2_vl (transformers 5.15.0; the reference's pin, 4.57.0, is
+# not installed): target sizes, grids and the float32 pixel_values (as SHA-256 plus sampled rows) of seeded images.
+
+def _processor_vectors():
+    import importlib.util
+    from pathlib import Path
+
+    golden = Path(__file__).resolve().parent / "golden"
+    spec = importlib.util.spec_from_file_location("make_processor_vectors", golden / "make_processor_vectors.py")
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod, np.load(golden / "processor_vectors.npz")
+
+
+def _case_names():
+    return [c[0] for c in _processor_vectors()[0].CASES]
+
+
+@pytest.mark.parametrize("name", _case_names())
+def test_resize_and_patch_rows_equal_the_library_bit_for_bit(name):
+    import hashlib
+
+    from oracle import resize_oracle as ro
+
+    mod, vec = _processor_vectors()
+    seed, h, w, lo, hi = (int(x) for x in vec[f"{name}/recipe"])
+    img = mod.seeded_image(seed, h, w)
+    assert hashlib.sha256(img.tobytes()).hexdigest() == str(vec[f"{name}/input_sha256"])
+    th, tw = ro.smart_resize(h, w, 28, lo, hi)
+    grid = vec[f"{name}/grid_thw"]
+    assert grid.tolist() == [[1, th // 14, tw // 14]]
+    resized = img if (th, tw) == (h, w) else ro.pil_resize(img, th, tw, ro.BICUBIC)
+    rows, g = po.patchify(resized[None])
+    assert list(g) == grid[0].tolist() and rows.dtype == np.float32
+    sample = vec[f"{name}/sample_rows"]
+    assert np.array_equal(rows[sample], vec[f"{name}/sample_values"])
+    assert hashlib.sha256(np.ascontiguousarray(rows).tobytes()).hexdigest() == str(vec[f"{name}/pixel_values_sha256"])
+
+
+def test_smart_resize_equals_the_library_on_its_table():
+    from oracle import resize_oracle as ro
+
+    table = _processor_vectors()[1]["smart_resize_table"]
+    assert len(table) >= 300
+    for h, w, lo, hi, th, tw in table.tolist():
+        assert ro.smart_resize(h, w, 28, lo, hi) == (th, tw), (h, w, lo, hi)
+
+
+def test_processor_vectors_discriminate():
+    """A plausible mistake in the oracle must fail the vectors: truncating instead of rounding the rescale, or the
+    bilinear filter in place of the bicubic one."""
+    from oracle import resize_oracle as ro
+
+    mod, vec = _processor_vectors()
+    name = "round_to_28_300x500"
+    seed, h, w, lo, hi = (int(x) for x in vec[f"{name}/recipe"])
+    img = mod.seeded_image(seed, h, w)
+    th, tw = ro.smart_resize(h, w, 28, lo, hi)
+    sample = vec[f"{name}/sample_rows"]
+    wrong_filter, _ = po.patchify(ro.pil_resize(img, th, tw, ro.BILINEAR)[None])
+    assert not np.array_equal(wrong_filter[sample], vec[f"{name}/sample_values"])
+    resized = ro.pil_resize(img, th, tw, ro.BICUBIC)
+
+    def rescale_in_float32(frames_u8, mean=po.OPENAI_CLIP_MEAN, std=po.OPENAI_CLIP_STD, scale=1.0 / 255.0):
+        x = frames_u8.astype(np.float32) * np.float32(scale)  # the library multiplies in float64 and rounds once
+        return (x - np.asarray(mean, dtype=np.float32)) / np.asarray(std, dtype=np.float32)
+
+    right = po.normalise
+    try:
+        po.normalise = rescale_in_float32
+        wrong_rescale, _ = po.patchify(resized[None])
+    finally:
+        po.normalise = right
+    assert not np.array_equal(wrong_rescale[sample], vec[f"{name}/sample_values"])
+    good, _ = po.patchify(resized[None])
+    assert np.array_equal(good[sample], vec[f"{name}/sample_values"])
