@@ -33,6 +33,10 @@ typedef void* mvit_stream_t; /* hipStream_t */
 enum { MVIT_F32 = 0, MVIT_BF16 = 1 };
 enum { MVIT_OK = 0, MVIT_ERR_ARG = -1, MVIT_ERR_LAUNCH = -2, MVIT_ERR_UNSUPPORTED = -3 };
 
+/* 200: mvit_attn_bwd takes the size of its workspace (delta_elems) and checks that outputs and inputs are disjoint;
+ *      mvit_adam_tensor rows are 96 bytes (shadow copy fields).  A caller built against an older header must be
+ *      rebuilt: compare mvit_version() with the value the header was written for. */
+#define MVIT_VERSION 200
 int mvit_version(void);
 const char* mvit_last_error(void);
 
@@ -164,8 +168,9 @@ typedef struct mvit_gemm_args {
   int64_t workspace_bytes;
   int split_k;   /* <= 1: one work-group per tile walks all of K.  > 1 (EPI_NONE, EPI_BIAS, EPI_BIAS_RES): K is cut in
                     split_k slices whose fp32 partial tiles go to `workspace`; a second kernel sums them in a fixed
-                    order and applies the epilogue (few output tiles, long contraction: weight gradients, and every
-                    GEMM of a batch of a few hundred patches) */
+                    order and applies the epilogue (few output tiles, long contraction).  Available to any caller; the
+                    vision tower uses it for weight gradients only, because a slice count chosen from M would make a
+                    row's result depend on how many rows share its batch */
 } mvit_gemm_args;
 
 /* C[M,N] = epilogue(sum_k A[m,k] * B[n,k]).  Operands must be 16-byte aligned with lda/ldb multiples of
@@ -189,11 +194,15 @@ int mvit_attn_fwd(const void* q, const void* k, const void* v, void* o, float* l
                   int64_t k_stride, int64_t v_stride, int64_t o_stride, float scale, int dtype,
                   mvit_stream_t stream);
 
-/* Gradients of the above.  delta: fp32 workspace [3, nheads, total] (row sums of o * d_o and two rescaled copies
- * of the row statistics).  dq/dk/dv use the strides given and must not overlap any input: the dq buffer is also
- * used as scratch (pre-scaled queries) before the result is written to it. */
+/* Gradients of the above.  delta: fp32 workspace of delta_elems floats; the call needs
+ * mvit_attn_bwd_delta_elems(...) of them ([nheads, total] row sums of o * d_o, and for bf16 / head_dim 80 /
+ * max_seqlen >= 512 two rescaled copies of the row statistics behind them) and refuses a shorter one.  dq/dk/dv use
+ * the strides given and must not overlap any input (checked on the host, MVIT_ERR_ARG): the dq buffer is also used as
+ * scratch (pre-scaled queries) before the result is written to it.
+ * Replaces the autograd of the attention-backend call, modeling:427-468 and :664-731. */
+int64_t mvit_attn_bwd_delta_elems(int max_seqlen, int64_t total, int nheads, int head_dim, int dtype);
 int mvit_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
-                  void* dq, void* dk, void* dv, float* delta, const int32_t* cu_seqlens,
+                  void* dq, void* dk, void* dv, float* delta, int64_t delta_elems, const int32_t* cu_seqlens,
                   const int32_t* seg_order, int n_seg, int max_seqlen, int64_t total, int nheads, int head_dim, int64_t q_stride, int64_t k_stride,
                   int64_t v_stride, int64_t o_stride, int64_t do_stride, int64_t dq_stride, int64_t dk_stride,
                   int64_t dv_stride, float scale, int dtype, mvit_stream_t stream);
@@ -333,7 +342,9 @@ int mvit_patch_embed_frames(const mvit_image* images, int n_images, int64_t tota
  * the horizontal pass (outer = frames * height, inner = 3) into an intermediate image followed by the vertical pass
  * (outer = frames, inner = new_width * 3); a pass whose size does not change is skipped by the caller.  bounds and kk
  * are device arrays that the host computes once per (in_len, out_len, filter) as Resample.c precompute_coeffs +
- * normalize_coeffs_8bpc do (Python: mi355_vit.pixels.resample_coefficients).
+ * normalize_coeffs_8bpc do (Python: mi355_vit.pixels.resample_coefficients).  Contract for tables of the caller's
+ * own: 0 <= bounds[2x], 0 <= bounds[2x + 1] <= ksize and bounds[2x] + bounds[2x + 1] <= in_len for every x; the device
+ * arrays are not read back to check it, the kernels force every window into that range instead.
  * Replaces, for frames that are already on the GPU, the two PIL resizes in front of the patch rows: the reference's
  * own fixed-size BILINEAR resize (python/data/preprocessing.py:126-131) and the BICUBIC resize to the smart_resize
  * target inside the image processor (transformers 4.57.0 Qwen2VLImageProcessor, reached through

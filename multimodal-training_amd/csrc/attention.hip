@@ -2258,9 +2258,29 @@ int check_common(const char* who, const int32_t* cu, int n_seg, int max_seqlen, 
   return MVIT_OK;
 }
 
+// Do two sets of `rows` rows of `width` bytes, starting at a and b with row pitches pa and pb (bytes), share a byte?
+// Exact when the pitches are equal (tensors interleaved in one buffer, like q | k | v, are told apart); otherwise the
+// two address ranges are compared as wholes.
+bool strided_rows_overlap(const void* a, int64_t pa, const void* b, int64_t pb, int64_t rows, int64_t width) {
+  const int64_t x = (int64_t)reinterpret_cast<uintptr_t>(a), y = (int64_t)reinterpret_cast<uintptr_t>(b);
+  const int64_t ea = x + (rows - 1) * pa + width, eb = y + (rows - 1) * pb + width;
+  if (ea <= y || eb <= x) return false;
+  if (pa != pb || pa < width) return true;
+  // equal pitch: row i of a starts at x + i*pa; relative to b's rows the column offset is constant
+  int64_t off = (x - y) % pa;
+  if (off < 0) off += pa;
+  // a's row covers [off, off + width) modulo the pitch; b's rows cover [0, width)
+  return off < width || off + width > pa;
+}
+
 }  // namespace
 
 extern "C" {
+
+int64_t mvit_attn_bwd_delta_elems(int max_seqlen, int64_t total, int nheads, int head_dim, int dtype) {
+  const bool wide = dtype == MVIT_BF16 && head_dim == 80 && max_seqlen >= WIDE_MIN_SEQLEN;
+  return (wide ? 3 : 1) * (int64_t)nheads * total;
+}
 
 int mvit_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* cu_seqlens,
                   const int32_t* seg_order, int n_seg, int max_seqlen, int64_t total, int nheads, int head_dim, int64_t q_stride, int64_t k_stride,
@@ -2290,7 +2310,7 @@ int mvit_attn_fwd(const void* q, const void* k, const void* v, void* o, float* l
 }
 
 int mvit_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse, void* dq,
-                  void* dk, void* dv, float* delta, const int32_t* cu_seqlens, const int32_t* seg_order, int n_seg, int max_seqlen,
+                  void* dk, void* dv, float* delta, int64_t delta_elems, const int32_t* cu_seqlens, const int32_t* seg_order, int n_seg, int max_seqlen,
                   int64_t total, int nheads, int head_dim, int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
                   int64_t do_stride, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride, float scale, int dtype,
                   mvit_stream_t stream) {
@@ -2298,6 +2318,21 @@ int mvit_attn_bwd(const void* q, const void* k, const void* v, const void* o, co
                             {q_stride, k_stride, v_stride, o_stride, do_stride, dq_stride, dk_stride, dv_stride},
                             {q, k, v, o, d_o, (const void*)lse, dq, dk, dv, (const void*)delta}))
     return rc;
+  if (total == 0) return MVIT_OK;
+  // the long-segment kernels keep three arrays of row statistics in the workspace and park the pre-scaled queries in dq
+  const bool wide = dtype == MVIT_BF16 && head_dim == 80 && max_seqlen >= WIDE_MIN_SEQLEN;
+  const int64_t need = (wide ? 3 : 1) * (int64_t)nheads * total;
+  MVIT_REQUIRE(delta_elems >= need, "attn_bwd: the delta workspace holds %lld floats, this call needs %lld (%d x nheads x total)",
+               (long long)delta_elems, (long long)need, wide ? 3 : 1);
+  {
+    const int64_t e = dtype == MVIT_BF16 ? 2 : 4, width = (int64_t)nheads * head_dim * e;
+    const struct { const void* ptr; int64_t stride; const char* name; } ins[] = {{q, q_stride, "q"}, {k, k_stride, "k"}, {v, v_stride, "v"}, {o, o_stride, "o"}, {d_o, do_stride, "d_o"}};
+    const struct { const void* ptr; int64_t stride; const char* name; } outs[] = {{dq, dq_stride, "dq"}, {dk, dk_stride, "dk"}, {dv, dv_stride, "dv"}};
+    for (const auto& w : outs)
+      for (const auto& r : ins)
+        MVIT_REQUIRE(!strided_rows_overlap(w.ptr, w.stride * e, r.ptr, r.stride * e, total, width),
+                     "attn_bwd: %s overlaps %s (outputs are written, and dq is used as scratch, before all inputs have been read)", w.name, r.name);
+  }
   if (n_seg == 0 || max_seqlen == 0 || total == 0) return MVIT_OK;
   AttnParams p = {};
   p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.lse = const_cast<float*>(lse); p.delta = delta;

@@ -1306,7 +1306,10 @@ int launch(const GemmParams& p, hipStream_t stream) {
   const size_t staging = (size_t)(BM / W::WM) * 32 * (BN + 8) * sizeof(float);
   const size_t lds = operands > staging ? operands : staging;
   auto kern = gemm_kernel<T, TO, TA, TB, EPI, VAR>;
-  static bool attr_set = false;  // dynamic LDS above 64 KiB needs opting in once per kernel
+  static bool attr_set_on[MVIT_MAX_DEVICES] = {};  // dynamic LDS above 64 KiB needs opting in once per kernel and device
+  const int dev = mvit_current_device("gemm");
+  if (dev < 0) return MVIT_ERR_LAUNCH;
+  bool& attr_set = attr_set_on[dev];
   if (!attr_set && lds > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return mvit_set_error(MVIT_ERR_LAUNCH, "gemm: hipFuncSetAttribute(%zu B LDS): %s", lds, hipGetErrorString(e));
@@ -1334,7 +1337,10 @@ int launch_dl(const GemmParams& p, hipStream_t stream) {
   constexpr size_t lds = staging_end > operands ? staging_end : operands;
   static_assert(lds <= 160 * 1024, "operand stages plus the epilogue staging area exceed the LDS of a CU");
   auto kern = gemm_dl_kernel<TO, TA, TB, EPI, NSTAGE, NW, MI16, PIX>;
-  static bool attr_set = false;
+  static bool attr_set_on[MVIT_MAX_DEVICES] = {};  // once per kernel and device
+  const int dev = mvit_current_device("gemm");
+  if (dev < 0) return MVIT_ERR_LAUNCH;
+  bool& attr_set = attr_set_on[dev];
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return mvit_set_error(MVIT_ERR_LAUNCH, "gemm: hipFuncSetAttribute(%zu B LDS): %s", lds, hipGetErrorString(e));
@@ -1342,10 +1348,11 @@ int launch_dl(const GemmParams& p, hipStream_t stream) {
   }
   if (p.split_k > 1 && EPI != MVIT_EPI_NONE) return mvit_set_error(MVIT_ERR_UNSUPPORTED, "gemm: split_k needs EPI_NONE");
   const int total = p.tiles_m * p.tiles_n * p.split_k;
-  static int n_cu = 0;
+  static int n_cu_on[MVIT_MAX_DEVICES] = {};  // persistent work-groups: one per compute unit of the launching device
+  int& n_cu = n_cu_on[dev];
   if (n_cu == 0) {
-    int dev = 0, v = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
     n_cu = v / 8 * 8 > 0 ? v / 8 * 8 : 8;
   }
   const int want = ((total + 7) / 8) * 8;

@@ -38,6 +38,20 @@ int mvit_set_error(int code, const char* fmt, ...);
 
 static inline bool mvit_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Per-device host state (function attributes set, compute-unit counts, symbol addresses) is kept in arrays of this
+// many slots indexed by the current device's ordinal.
+#define MVIT_MAX_DEVICES 64
+// Ordinal of the current device, or -1 (with the error recorded) when it cannot be told or has no slot.
+static inline int mvit_current_device(const char* who) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= MVIT_MAX_DEVICES) {
+    mvit_set_error(MVIT_ERR_LAUNCH, "%s: hipGetDevice: %s (device %d, %d slots)", who, hipGetErrorString(e), dev, MVIT_MAX_DEVICES);
+    return -1;
+  }
+  return dev;
+}
+
 template <typename T>
 struct mvit_elem;
 template <>

@@ -229,16 +229,22 @@ int check_table(const char* what, const mvit_adam_tensor* tensors, int n_tensors
   return MVIT_OK;
 }
 
-constexpr int MAX_DEVICES = 64;
 std::mutex g_scratch_mutex;
-float* g_scratch_ptr[MAX_DEVICES] = {};  // device address of `scratch` on each device, looked up on first use
+float* g_scratch_ptr[MVIT_MAX_DEVICES] = {};  // device address of `scratch` on each device, looked up on first use
 
-// Address of the current device's copy of `scratch` (set-up on the first call per device; no allocation).
-int static_scratch(float** out) {
-  int dev = -1;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES)
-    return mvit_set_error(MVIT_ERR_LAUNCH, "grad_sumsq_static: hipGetDevice: %s (device %d)", hipGetErrorString(e), dev);
+// Address of `scratch` on the device that owns `stream` (set-up on the first call per device; no allocation).  The
+// launch goes to the current device, so a stream of another device is refused instead of being handed this one's array.
+int static_scratch(float** out, hipStream_t stream) {
+  const int dev = mvit_current_device("grad_sumsq_static");
+  if (dev < 0) return MVIT_ERR_LAUNCH;
+  hipError_t e = hipSuccess;
+  if (stream != nullptr) {
+    hipDevice_t sdev = -1;
+    e = hipStreamGetDevice(stream, &sdev);
+    if (e != hipSuccess || (int)sdev != dev)
+      return mvit_set_error(MVIT_ERR_ARG, "grad_sumsq_static: the stream belongs to device %d, the current device is %d (%s)", (int)sdev, dev,
+                            hipGetErrorString(e));
+  }
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (g_scratch_ptr[dev] == nullptr) {
     void* p = nullptr;
@@ -300,7 +306,7 @@ int mvit_grad_sumsq_static(const mvit_adam_tensor* tensors, int n_tensors, int64
                "grad_sumsq_static: %lld chunks exceed the built-in scratch of %d chunks (%lld elements); use mvit_grad_sumsq with a workspace",
                (long long)n_chunks, MVIT_SUMSQ_STATIC_MAX_CHUNKS, (long long)MVIT_SUMSQ_STATIC_MAX_CHUNKS * MVIT_ADAM_CHUNK);
   float* partial = nullptr;
-  if (int rc = static_scratch(&partial)) return rc;
+  if (int rc = static_scratch(&partial, reinterpret_cast<hipStream_t>(stream))) return rc;
   // every partial in [0, n_chunks) is overwritten by the first kernel, so nothing has to be cleared between calls
   return mvit_grad_sumsq(tensors, n_tensors, n_chunks, partial, out, dtype, stream);
 }

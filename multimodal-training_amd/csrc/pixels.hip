@@ -107,6 +107,18 @@ __global__ __launch_bounds__(256) void patchify_kernel(const mvit_image* __restr
 }
 
 }  // namespace
+// A window as the kernels use it: first tap and tap count forced into the table's row (ksize entries) and into the
+// input axis, so that a table that breaks the entry point's contract cannot make a kernel read outside its arrays.
+struct TapWindow {
+  int xmin, n;
+};
+__device__ __forceinline__ TapWindow tap_window(const int32_t* __restrict__ bounds, int64_t x, int ksize, int64_t in_len) {
+  int xmin = bounds[2 * x], n = bounds[2 * x + 1];
+  xmin = max(0, min(xmin, (int)in_len - 1));
+  n = max(0, min(n, min(ksize, (int)in_len - xmin)));
+  return {xmin, n};
+}
+
 
 // ------------------------------------------------------------------------------------------------
 // One resampling pass along the middle axis of a uint8 array [outer][in_len][inner] -> [outer][out_len][inner], with
@@ -134,7 +146,8 @@ __global__ __launch_bounds__(256) void resample_pass_kernel(const uint8_t* __res
     uint8_t* d = dst + o * row_out + 4 * q;
     if (WIDE) {
       const int64_t x = (4 * q) / inner, c = (4 * q) % inner;
-      const int xmin = bounds[2 * x], n = bounds[2 * x + 1];
+      const TapWindow tw = tap_window(bounds, x, ksize, in_len);
+      const int xmin = tw.xmin, n = tw.n;
       const int32_t* k = kk + x * ksize;
       int a0 = 1 << (RESAMPLE_PRECISION_BITS - 1), a1 = a0, a2 = a0, a3 = a0;
       for (int t = 0; t < n; ++t) {
@@ -151,7 +164,8 @@ __global__ __launch_bounds__(256) void resample_pass_kernel(const uint8_t* __res
         const int64_t e = 4 * q + b;
         if (e >= row_out) break;
         const int64_t x = e / inner, c = e % inner;
-        const int xmin = bounds[2 * x], n = bounds[2 * x + 1];
+        const TapWindow tw = tap_window(bounds, x, ksize, in_len);
+      const int xmin = tw.xmin, n = tw.n;
         const int32_t* k = kk + x * ksize;
         int a = 1 << (RESAMPLE_PRECISION_BITS - 1);
         for (int t = 0; t < n; ++t) a += (int)s[(int64_t)(xmin + t) * inner + c] * k[t];
@@ -195,7 +209,8 @@ __global__ __launch_bounds__(256) void resample_rows_lds_kernel(const uint8_t* _
     uint8_t* d = dst + o * row_out;
     // a thread makes whole pixels: the channels of a pixel share its window and its weights
     for (int x = threadIdx.x; x < (int)out_len; x += 256) {
-      const int xmin = bounds[2 * x], n = bounds[2 * x + 1];
+      const TapWindow tw = tap_window(bounds, x, ksize, in_len);
+      const int xmin = tw.xmin, n = tw.n;
       const int32_t* k = kk + (int64_t)x * ksize;
       int acc[RESAMPLE_MAX_CHANNELS];
 #pragma unroll
@@ -231,7 +246,8 @@ __global__ __launch_bounds__(256) void resample_cols_kernel(const uint8_t* __res
   const int x_first = blockIdx.x * 256, x_last = min(x_first + 255, (int)out_len - 1);
   const bool mine = x_first + (int)threadIdx.x <= x_last;
   const int x = mine ? x_first + (int)threadIdx.x : x_last;
-  const int xmin = bounds[2 * x], n = bounds[2 * x + 1];
+  const TapWindow tw = tap_window(bounds, x, ksize, in_len);
+      const int xmin = tw.xmin, n = tw.n;
   int k[RESAMPLE_KMAX];
 #pragma unroll
   for (int t = 0; t < RESAMPLE_KMAX; ++t) k[t] = t < n ? kk[(int64_t)x * ksize + t] : 0;

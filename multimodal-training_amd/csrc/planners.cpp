@@ -21,7 +21,7 @@ int mvit_set_error(int code, const char* fmt, ...) {
 
 extern "C" {
 
-int mvit_version(void) { return 100; }
+int mvit_version(void) { return MVIT_VERSION; }
 const char* mvit_last_error(void) { return g_err; }
 
 static int check_grid(const int64_t* g, int64_t n, int merge) {

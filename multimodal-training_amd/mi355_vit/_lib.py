@@ -82,9 +82,10 @@ PROTOTYPES = {
     "mvit_resample_u8": [_vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _i32, _vp],
     "mvit_patch_embed_pack_weight": [_vp, _i32, _i64, _i64, _vp, _vp],
     "mvit_patch_embed_frames": [_vp, _i32, _i64, _vp, _i64, _vp, _i64, _i32, C.c_double] + [_f32] * 6 + [_vp],
-    "mvit_attn_bwd": [_vp] * 12 + [_i32, _i32, _i64, _i32, _i32] + [_i64] * 8 + [_f32, _i32, _vp],
+    "mvit_attn_bwd": [_vp] * 10 + [_i64, _vp, _vp] + [_i32, _i32, _i64, _i32, _i32] + [_i64] * 8 + [_f32, _i32, _vp],
 }
-EXPORTS = sorted(list(PROTOTYPES) + ["mvit_version", "mvit_last_error"])
+EXPORTS = sorted(list(PROTOTYPES) + ["mvit_version", "mvit_last_error", "mvit_attn_bwd_delta_elems"])
+HEADER_VERSION = 200  # MVIT_VERSION of include/mi355_vit.h these prototypes were written for
 
 _lib = None
 
@@ -107,6 +108,10 @@ def load() -> C.CDLL:
         lib.mvit_version.restype = C.c_int
         lib.mvit_last_error.argtypes = []
         lib.mvit_last_error.restype = C.c_char_p
+        lib.mvit_attn_bwd_delta_elems.argtypes = [_i32, _i64, _i32, _i32, _i32]
+        lib.mvit_attn_bwd_delta_elems.restype = _i64
+        if lib.mvit_version() != HEADER_VERSION:
+            raise RuntimeError(f"{LIB_PATH} reports interface version {lib.mvit_version()}, these bindings are written for {HEADER_VERSION}: rebuild the library")
         _lib = lib
     return _lib
 

@@ -238,7 +238,8 @@ def segment_copy(src: torch.Tensor, dst: torch.Tensor, segments: Sequence[Tuple[
             raise ValueError(f"segment_copy: segment ({a},{b},{n}) out of bounds for {src.shape[0]} -> {dst.shape[0]} rows")
     if not segs:
         return dst
-    desc = torch.tensor(segs, dtype=torch.int64).to(src.device, non_blocking=False)
+    # pinned staging + asynchronous copy: the launch below is ordered behind it on the same stream, the host does not wait
+    desc = torch.tensor(segs, dtype=torch.int64).pin_memory().to(src.device, non_blocking=True)
     row_bytes = src.shape[1] * src.element_size()
     rc = _lib.load().mvit_segment_copy(src.data_ptr(), dst.data_ptr(), desc.data_ptr(), len(segs), max(n for _, _, n in segs), row_bytes, _stream(src))
     _lib.check(rc, "mvit_segment_copy")
@@ -255,7 +256,7 @@ def pad_pack(pack: torch.Tensor, lens: Sequence[int], pad_len: int, pad_value: f
     for n in lens:
         offs.append(o)
         o += n
-    meta = torch.tensor([list(lens), offs], dtype=torch.int64).to(pack.device)
+    meta = torch.tensor([list(lens), offs], dtype=torch.int64).pin_memory().to(pack.device, non_blocking=True)
     padded = torch.empty(B, pad_len, pack.shape[1], dtype=pack.dtype, device=pack.device)
     mask = torch.empty(B, pad_len, dtype=torch.uint8, device=pack.device)
     bits = torch.tensor([pad_value], dtype=pack.dtype).view(torch.int16 if pack.element_size() == 2 else torch.int32).item() & (0xFFFF if pack.element_size() == 2 else 0xFFFFFFFF)
@@ -367,8 +368,8 @@ _N_CU = 256  # MI355X compute units; one 256x256 GEMM work-group runs per CU
 @functools.lru_cache(maxsize=None)
 def wgrad_split_k(out_rows: int, out_cols: int, k: int) -> int:
     """K slices for a GEMM with few output tiles (256x256) and a long contraction: the weight gradients (contraction
-    over the tokens) at any batch size, and the forward / input-gradient GEMMs of a small batch (a few hundred to a few
-    thousand patches give 5 to 80 tiles for 256 compute units; from about 25,000 patches on the answer is 1).
+    over the tokens).  The model uses it for those only: on a forward or input-gradient GEMM a slice count chosen
+    from the batch size would make a row's result depend on how many rows share its batch.
 
     Picks the slice count with the lowest modelled time.  Work items (tiles x slices) run in rounds of one per
     CU, so the count should fill whole rounds; every slice costs an fp32 partial tile that a second kernel
@@ -389,9 +390,6 @@ def wgrad_split_k(out_rows: int, out_cols: int, k: int) -> int:
         if best_t is None or t < best_t:
             best, best_t = sk, t
     return best
-
-
-split_k_for = wgrad_split_k  # the same model, under the name the forward and input-gradient GEMMs call it by
 
 
 # ------------------------------------------------------------------------------ attention
@@ -477,12 +475,13 @@ def attn_bwd(q, k, v, o, d_o, lse, cu_seqlens, max_seqlen, nheads, head_dim, sca
             raise ValueError("attn_bwd: row count / dtype mismatch")
     if tuple(lse.shape) != (nheads, S) or lse.dtype != torch.float32 or not lse.is_contiguous():
         raise ValueError("attn_bwd: lse must be contiguous fp32 [nheads, S]")
-    delta = torch.empty(3, nheads, S, dtype=torch.float32, device=q.device)  # workspace: delta, -lse*log2(e), -delta
+    # workspace: delta, and for the long-segment kernels -lse*log2(e) and -delta behind it
+    delta = torch.empty(_lib.load().mvit_attn_bwd_delta_elems(max_seqlen, S, nheads, head_dim, dt(q)), dtype=torch.float32, device=q.device)
     st = _stream(q)
     strides = tuple(_attn_view(t, nheads, head_dim, nm) for t, nm in ((q, "q"), (k, "k"), (v, "v"), (o, "o"), (d_o, "do"), (dq, "dq"), (dk, "dk"), (dv, "dv")))
     rc = _launch("attn_bwd", {"cu": cu_seqlens, "max_seqlen": max_seqlen, "nheads": nheads, "head_dim": head_dim}, lambda: _lib.load().mvit_attn_bwd(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(), lse.data_ptr(),
-        dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(), cu_seqlens.data_ptr(), order_ptr,
+        dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(), delta.numel(), cu_seqlens.data_ptr(), order_ptr,
         cu_seqlens.numel() - 1, max_seqlen, S, nheads, head_dim, *strides, scale, dt(q), st))
     _lib.check(rc, "mvit_attn_bwd")
     return dq, dk, dv

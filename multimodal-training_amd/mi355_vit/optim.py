@@ -15,6 +15,7 @@ from __future__ import annotations
 
 import ctypes as C
 import math
+import os
 from typing import Dict, Iterable, List, Optional, Tuple
 
 import numpy as np
@@ -39,7 +40,23 @@ def attach_shadow(param: torch.Tensor, copy: torch.Tensor) -> None:
         raise ValueError("attach_shadow: the copy must be a 1-D / 2-D unit-stride view of the parameter's shape on its device")
     if copy.dtype not in (param.dtype, torch.bfloat16):
         raise ValueError("attach_shadow: the copy's dtype must be the parameter's or bfloat16")
+    global _SHADOW_GENERATION
     param._mvit_shadow = copy
+    _SHADOW_GENERATION += 1  # every plan built before this call is stale
+
+
+_SHADOW_GENERATION = 0
+
+
+def check_shadows(params) -> None:
+    """Debug aid (``MVIT_CHECK_SHADOWS=1`` runs it before every step): every operand copy must equal its parameter,
+    cast to the copy's dtype.  A writer that updates parameters through raw pointers without storing the copy too
+    (another fused optimizer, a custom kernel) leaves the copies stale with no version bump; this is what finds it."""
+    for p in params:
+        sh = getattr(p, "_mvit_shadow", None)
+        if sh is not None and not torch.equal(sh, p.detach().to(sh.dtype)):
+            raise RuntimeError(f"operand copy of a parameter of shape {tuple(p.shape)} differs from the parameter: something updated it "
+                               "through a raw pointer without storing the copy (see attach_shadow)")
 
 
 def _shadow_fields(p: torch.Tensor) -> tuple:
@@ -156,7 +173,9 @@ class FusedAdam(torch.optim.Adam):
                 loss = closure()
         # which parameters take part (those with a gradient) and where they and their moments live rarely changes:
         # the table is rebuilt only when it does; per step only gradient addresses and scalars are refreshed
-        key = tuple((id(p), p.data_ptr(), _shadow_fields(p)) for group in self.param_groups for p in group["params"] if p.grad is not None)
+        key = (_SHADOW_GENERATION, tuple((id(p), p.data_ptr()) for group in self.param_groups for p in group["params"] if p.grad is not None))
+        if os.environ.get("MVIT_CHECK_SHADOWS") == "1":
+            check_shadows(p for group in self.param_groups for p in group["params"])
         stale = key != self._plan_key or any(
             int(bk.step_tensors[0].item()) != int(bk.steps[0]) or int(bk.step_tensors[-1].item()) != int(bk.steps[-1])
             for bk in self._plan)  # step counters edited from outside (cheap spot check of the host mirror)

@@ -21,8 +21,40 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.mvit_version() >= 100
+    assert lib.mvit_version() == _lib.HEADER_VERSION == int(re.search(r"#define MVIT_VERSION (\d+)", header).group(1))
     assert isinstance(lib.mvit_last_error(), bytes)
+
+
+def test_attention_backward_refuses_a_short_workspace_and_overlapping_buffers():
+    """Host-side argument checks of mvit_attn_bwd: they return before anything is launched, so made-up (aligned,
+    never dereferenced) addresses are enough and no GPU is needed."""
+    from mi355_vit import _lib
+
+    lib = _lib.load()
+    S, H, d = 1024, 16, 80
+    C3 = 3 * H * d
+    qkv, dqkv, o, do, lse, delta, cu = 0x10000000, 0x20000000, 0x30000000, 0x38000000, 0x40000000, 0x48000000, 0x50000000
+    e = 2  # bf16
+    need = lib.mvit_attn_bwd_delta_elems(S, S, H, d, _lib.BF16)
+    assert need == 3 * H * S and lib.mvit_attn_bwd_delta_elems(64, S, H, d, _lib.BF16) == H * S
+    assert lib.mvit_attn_bwd_delta_elems(S, S, H, d, _lib.F32) == H * S
+
+    def call(dq=dqkv, dk=dqkv + H * d * e, dv=dqkv + 2 * H * d * e, n_delta=need, dq_stride=C3):
+        # n_seg = 0: the checks run, a call that passes them launches nothing (the addresses are made up)
+        return lib.mvit_attn_bwd(qkv, qkv + H * d * e, qkv + 2 * H * d * e, o, do, lse, dq, dk, dv, delta, n_delta, cu, None, 0, S, S, H, d,
+                                 C3, C3, C3, H * d, H * d, dq_stride, C3, C3, 1.0, _lib.BF16, None)
+
+    assert call(n_delta=need - 1) == -1 and b"delta workspace" in lib.mvit_last_error()
+    assert call(dq=qkv) == -1 and b"dq overlaps q" in lib.mvit_last_error()  # in place on the queries
+    assert call(dq=qkv + 8 * e) == -1 and b"dq overlaps" in lib.mvit_last_error()  # shifted by a few columns
+    assert call(dk=o, dq_stride=C3) == -1 and b"dk overlaps o" in lib.mvit_last_error()
+    assert call() == 0
+    # rows interleaved with the inputs in one buffer but on other columns are disjoint and pass the check
+    wide_pitch = 2 * C3
+    rc = lib.mvit_attn_bwd(qkv, qkv + H * d * e, qkv + 2 * H * d * e, o, do, lse, qkv + C3 * e, qkv + C3 * e + H * d * e, qkv + C3 * e + 2 * H * d * e,
+                           delta, need, cu, None, 0, S, S, H, d, wide_pitch, wide_pitch, wide_pitch, H * d, H * d, wide_pitch, wide_pitch, wide_pitch,
+                           1.0, _lib.BF16, None)
+    assert rc == 0, lib.mvit_last_error()  # no segments: the arguments pass the checks and nothing is launched
 
 
 def test_gemm_args_struct_matches_header_field_order():

@@ -35,8 +35,12 @@ def test_static_scratch_sum_of_squares_equals_the_workspace_entry_point(dtype):
         ref = torch.zeros(1, dtype=torch.float64, device=DEV)
         out = torch.zeros(1, dtype=torch.float64, device=DEV)
         _lib.check(lib.mvit_grad_sumsq(table.data_ptr(), n, n_chunks, partial.data_ptr(), ref.data_ptr(), code, stream), "mvit_grad_sumsq")
+        # the call itself takes no device memory: the driver's free-memory figure is the same before and after it
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
         _lib.check(lib.mvit_grad_sumsq_static(table.data_ptr(), n, n_chunks, out.data_ptr(), code, stream), "mvit_grad_sumsq_static")
         torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
         assert out.item() == ref.item() and out.item() > 0.0
         exact = sum(float(x.double().pow(2).sum()) for x in grads)
         assert abs(out.item() - exact) <= 1e-6 * exact
