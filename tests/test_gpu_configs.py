@@ -4,7 +4,7 @@ cfg2  depth-32 tower, bf16.  (a) The two smallest images of the seed-1 ragged ba
       and all 518 parameter gradients, printed per parameter kind next to the error of the oracle itself evaluated in
       bf16 (tests/golden/bf16_oracle_errors.json, written by tests/golden/make_bf16_oracle_errors.py): what a bf16 run
       of the reference's own arithmetic shows against fp32.  The bar per kind is
-      max(2e-2, 1.25 x the bf16 oracle's error for that kind) and the branch each kind took is printed.  (b) The whole
+      max(2e-2, 1.5 x the bf16 oracle's error for that kind) and the branch each kind took is printed.  (b) The whole
       eight-image batch (25,524 patches) through properties that need no O(L^2) host pass: finite, checkpointed == plain
       bit for bit, and batch == images run one at a time (outputs bit-equal row for row, parameter gradients equal
       to the sum of the single-image gradients within bf16 rounding of the sums).
@@ -80,7 +80,7 @@ def _kind(name):
 def _check_against_oracle_with_bf16_bar(tag, case):
     """Output <= 2e-2 in both metrics.  Gradients: per parameter kind (q / k / v / proj / gate / up / down weights and
     biases, norms, patch embedding, merger) the worst error over the 32 blocks against the same figure of the bf16
-    oracle; bar = max(2e-2, 1.25 x bf16 oracle), both metrics."""
+    oracle; bar = max(2e-2, 1.5 x bf16 oracle), both metrics."""
     fixture = json.loads((GOLDEN / "bf16_oracle_errors.json").read_text())[case["name"]]
     assert fixture["grid_thw"] == case["grid"].tolist()
     model = _build(case["kw"], case["seed"])
@@ -107,8 +107,8 @@ def _check_against_oracle_with_bf16_bar(tag, case):
     failures = []
     print(f"[{tag}] parameter gradients per kind, worst over the blocks: kernels vs fp32 oracle | bf16 oracle vs fp32 oracle | bar (branch)", flush=True)
     for k in sorted(mine, key=lambda k: -mine[k][0]):
-        bar_m, bar_f = max(2e-2, 1.25 * theirs[k][0]), max(2e-2, 1.25 * theirs[k][1])
-        branch = "2e-2" if bar_m == 2e-2 and bar_f == 2e-2 else "1.25 x bf16 oracle"
+        bar_m, bar_f = max(2e-2, 1.5 * theirs[k][0]), max(2e-2, 1.5 * theirs[k][1])
+        branch = "2e-2" if bar_m == 2e-2 and bar_f == 2e-2 else "1.5 x bf16 oracle"
         print(f"[{tag}]   {k:32s} max-rel {mine[k][0]:.3e} ({mine[k][2]}) frob {mine[k][1]:.3e} | {theirs[k][0]:.3e} {theirs[k][1]:.3e} | "
               f"{bar_m:.3e} {bar_f:.3e} ({branch})", flush=True)
         if not (mine[k][0] < bar_m and mine[k][1] < bar_f):
