@@ -4,7 +4,7 @@ vision tower (bf16).  Default workload: one 3584 x 3584 image = 65,536 patches w
 checkpointing (the largest single-GPU configuration); the 8-image ragged batch (cfg2) and the video (cfg5) are
 timed beside it and reported under "other_workloads".
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg5|cfg1|sample_yaml|one_224]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg5|cfg1|sample_yaml|one_896|one_224]
 
 One "step" = zero_grad, forward, backward with a fixed upstream gradient (the optimizer is not part of the
 path; "with_optimizer_step" reports the same loop with gradient norm, clipping and one Adam step added).  Inputs
@@ -59,6 +59,10 @@ def make_workload(name: str):
         # = 802,816 (896 x 896 px = 64 x 64 patches per image), bfloat16, activation checkpointing on
         return ("full tower, 4 images 896x896 = 16,384 patches, per-block activation checkpointing (the reference's sample.yaml)",
                 FULL_TOWER, torch.bfloat16, torch.tensor([[1, 64, 64]] * 4), 4, True)
+    if name == "one_896":
+        # the lower end of the batch sizes the reference's README names as usual (4-16 k tokens per step)
+        return ("full tower, one 896x896 image = 4,096 patches, per-block activation checkpointing",
+                FULL_TOWER, torch.bfloat16, torch.tensor([[1, 64, 64]]), 6, True)
     if name == "one_224":
         return ("full tower, one 224x224 image = 256 patches (a batch too small to fill the GPU: what a step costs at least)",
                 FULL_TOWER, torch.bfloat16, torch.tensor([[1, 16, 16]]), 5, False)
@@ -108,12 +112,21 @@ def summarise_trace(records, cfg_kw, dtype):
     return out
 
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, scaled by what the same
-# counters read for a 1 GiB device copy: x2.000 and x1.000), keyed by (workload, trace tag).  The weight-gradient
-# launch is the GEMM kernel (544.2 MB) plus its split-K reduction (98.4 MB).
-# The full-attention backward launch of cfg3 is the dK/dV kernel (4.91 GB read + 0.34 GB written) plus the dQ kernel
-# (4.84 GB + 0.17 GB) plus the two small preparation kernels (0.5 GB): profiles/attn_cfg3_pmc.txt.
-MEASURED_TRAFFIC_BYTES = {("cfg2", "gemm_tt_epi0"): 642.6e6, ("cfg3", "attn_bwd_full"): 10.8e9}
+def measured_traffic_bytes(workload: str, tag: str):
+    """HBM bytes per launch of a kernel group, as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs,
+    each scaled by what the same counter reads for a 1 GiB device copy).  The figures live with the counter summaries
+    they come from: a line ``traffic_bytes_per_launch <workload> <trace tag> <bytes>`` in a text file under profiles/.
+    None when no summary holds such a line."""
+    for f in sorted((ROOT / "profiles").glob("*.txt")):
+        for line in f.read_text().splitlines():
+            parts = line.split()
+            if len(parts) >= 4 and parts[0] == "traffic_bytes_per_launch" and parts[1] == workload and parts[2] == tag:
+                try:
+                    return float(parts[3])
+                except ValueError:
+                    return None
+    return None
+
 
 KERNEL_NAMES = {
     "gemm_nn_epi0": "gemm_dl_kernel<TO, TA=false, TB=false, EPI=NONE>",
@@ -334,8 +347,9 @@ def cpu_baseline(cfg_kw, grid, seed, dtype, budget_s: float = 30.0):
     from mi355_vit.config import Qwen2_5_VLVisionConfig
     from mi355_vit.modeling import Qwen2_5_VisionTransformerPretrainedModel
 
-    cores = min(16, os.cpu_count() or 1)
-    torch.set_num_threads(cores)
+    # every core this process may use: torch's default thread count follows OMP_NUM_THREADS (a GPU box gives a job its
+    # share of the host that way) and is the machine's core count otherwise
+    cores = torch.get_num_threads()
     order = sorted(range(grid.shape[0]), key=lambda i: int(grid[i].prod()))[:2]
     sub = grid[order].clone()
     sub[:, 0] = sub[:, 0].clamp(max=2)
@@ -371,7 +385,7 @@ def cpu_baseline(cfg_kw, grid, seed, dtype, budget_s: float = 30.0):
     n_full = len([i for i in cfg_kw["fullatt_block_indexes"] if i < cfg_kw["depth"]])
     if cfg_kw["depth"] < 2 or n_full == 0:
         t = timed(cfg_kw["depth"], list(cfg_kw["fullatt_block_indexes"]))
-        return {"value": S0 / t, "unit": "patches/s", "cores": cores, "kind": "port",
+        return {"value": S0 / t, "unit": "patches/s", "cores": cores, "host_cores_visible": os.cpu_count(), "kind": "port",
                 "sample": f"{S0} patches, whole tower fwd+bwd in fp32 took {t:.2f} s"}
     t_w = timed(1, [])      # patch embed + one windowed block + merger
     t_wf = timed(2, [1])    # ... + one full-attention block
@@ -383,6 +397,7 @@ def cpu_baseline(cfg_kw, grid, seed, dtype, budget_s: float = 30.0):
         "value": S / total,
         "unit": "patches/s",
         "cores": cores,
+        "host_cores_visible": os.cpu_count(),
         "kind": "port",
         "sample": f"grid {sub.tolist()} ({S0} patches) fwd+bwd in fp32: patch embed + 1 windowed block + merger {t_w:.2f} s, the same + 1 full block {t_wf:.2f} s; "
                   f"extrapolated to {cfg_kw['depth']} blocks ({n_full} full) of {S} patches: linear part x{lin:.2f}, full-attention excess "
@@ -442,17 +457,33 @@ def main() -> None:
         out = model(hidden_states=pixels, grid_thw=grid_dev)
         out.backward(gout)
 
-    def timed_steps(fn, warmup, steps):
+    def timed_steps(fn, warmup, steps, detail=None):
+        """Wall-clock time of `steps` calls between two synchronisations.  With `detail` (a dict) also: a pair of HIP
+        events on the compute stream around every call (the second stream joins the main one before a block hands
+        its gradients back, so the closing event covers both) and the time the host needs to issue the calls."""
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)] if detail is not None else None
         t0 = time.perf_counter()
-        for _ in range(steps):
+        for i in range(steps):
+            if pairs:
+                pairs[i][0].record()
             fn()
+            if pairs:
+                pairs[i][1].record()
+        t_issued = time.perf_counter()
         torch.cuda.synchronize()
-        return time.perf_counter() - t0
+        t1 = time.perf_counter()
+        if pairs:
+            per = sorted(a.elapsed_time(b) for a, b in pairs)
+            detail["event_ms_median"] = per[len(per) // 2] if len(per) % 2 else 0.5 * (per[len(per) // 2 - 1] + per[len(per) // 2])
+            detail["event_ms_min"], detail["event_ms_max"] = per[0], per[-1]
+            detail["host_issue_ms_per_step"] = 1000.0 * (t_issued - t0) / max(1, steps)
+        return t1 - t0
 
-    elapsed = timed_steps(step, args.warmup, args.steps)
+    timing = {}
+    elapsed = timed_steps(step, args.warmup, args.steps, timing)
     ms_per_step = 1000.0 * elapsed / max(1, args.steps)
     peak_mem_gb = torch.cuda.max_memory_allocated() / 2**30
 
@@ -475,7 +506,7 @@ def main() -> None:
             kernel_name = f"gemm_kernel<float, float, ...> ({dom})" if dom.startswith("gemm") else f"attn_*_f32 ({dom})"
         roofline = {"bound": "mfma", "kernel": kernel_name, "launches_per_step": d["launches"],
                     "avg_launch_ms": d["ms"] / d["launches"], "achieved": ach, "peak": peak, "unit": "TFLOP/s",
-                    "frac": ach / peak, "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, dom))}
+                    "frac": ach / peak, "traffic": measured_traffic_bytes(args.workload, dom)}
         a_ms = sum(v["ms"] for t, v in summ.items() if t.startswith("attn"))
         a_fl = sum(v["flops"] for t, v in summ.items() if t.startswith("attn"))
         attn_util = a_fl / (a_ms * 1e-3) / 1e12 / peak if a_ms > 0 else None
@@ -534,18 +565,20 @@ def main() -> None:
 
         torch.cuda.synchronize()
         torch.cuda.reset_peak_memory_stats()
+        det = {}
         try:
-            t = timed_steps(step2, 2, 5)
+            t = timed_steps(step2, 2, 5, det)
         finally:
             (model.gradient_checkpointing_enable if ckpt else model.gradient_checkpointing_disable)()
         return {"patches": S2, "grid_thw": grid2.tolist(), "activation_checkpointing": ckpt2, "steps": 5,
                 "ms_per_step": round(1000.0 * t / 5, 3), "patches_per_s": round(S2 / (t / 5), 1),
+                "event_ms_median": round(det["event_ms_median"], 3), "host_issue_ms_per_step": round(det["host_issue_ms_per_step"], 3),
                 "peak_mem_gb": round(torch.cuda.max_memory_allocated() / 2**30, 2)}
 
     optimizer = handoff = input_side = with_opt = None
     others = None
     if not args.no_other_workloads and cfg_kw == FULL_TOWER:
-        others = {name: side_leg(other_workload, name) for name in ("cfg2", "cfg3", "cfg5", "sample_yaml") if name != args.workload}
+        others = {name: side_leg(other_workload, name) for name in ("cfg2", "cfg3", "cfg5", "sample_yaml", "one_896") if name != args.workload}
         # the 65,536-patch image with every activation kept (no block is run twice): what 288 GB of HBM allow;
         # reported beside the metric, which stays on the configuration as it is named (checkpointing per block)
         others["cfg3_all_activations_kept"] = side_leg(other_workload, "cfg3", False)
@@ -567,6 +600,9 @@ def main() -> None:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
+        "timing": {"value_uses": "wall-clock mean of the timed steps between two synchronisations (ms_per_step)",
+                   "event_ms_median": round(timing["event_ms_median"], 3), "event_ms_min": round(timing["event_ms_min"], 3),
+                   "event_ms_max": round(timing["event_ms_max"], 3), "host_issue_ms_per_step": round(timing["host_issue_ms_per_step"], 3)},
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
