@@ -14,6 +14,8 @@
 // read and results written as 16-byte vectors along N.
 // Work-group ids are remapped so that the tiles a single XCD (one L2) works on are neighbours in N.
 #include "mvit_common.h"
+#include <math.h>
+#include <stdlib.h>
 #include <string.h>
 #include <type_traits>
 
@@ -853,11 +855,17 @@ __global__ __launch_bounds__(Waves<VAR>::NTHREADS, Waves<VAR>::MIN_WAVES) void g
 // Rows past the matrix edge are clamped to valid rows (they only feed outputs that are never stored).  A partial
 // last K tile (K not a multiple of 32) is loaded through registers with zeros past the end of K.
 // The compiler does not see these loads: s_waitcnt vmcnt is placed by hand (loads return in order).
-template <int NW>  // waves per work-group: 8 -> each owns 128x64 (two waves per SIMD), 4 -> 128x128 (one per SIMD)
+// waves per work-group: 8 -> each owns 128x64 (two waves per SIMD), 4 -> 128x128 (one per SIMD).  BM_ = 128: an output
+// tile of half the height for products whose 256-row tiles would leave most compute units idle: the eight waves own
+// 64x64 each, the A stage holds 128 rows (in the first half of its 16 KiB slot), everything an output element sees
+// (K order, MFMA form, epilogue arithmetic) is unchanged, so results are bit-identical to the 256-row tile's.
+template <int NW, int BM_ = 256>
 struct DL {
-  static constexpr int BM = 256, BN = 256, BK = 32, WM = 128, WN = NW == 8 ? 64 : 128, NTHREADS = 64 * NW;
+  static_assert(BM_ == 256 || (BM_ == 128 && NW == 8), "tile heights built: 256, and 128 with eight waves");
+  static constexpr int BM = BM_, BN = 256, BK = 32, WM = BM_ / 2, WN = NW == 8 ? 64 : 128, NTHREADS = 64 * NW;
   static constexpr int TILE_BYTES = 256 * BK * 2;
-  static constexpr int CPT = 16 / NW;  // 1 KiB load instructions per wave, operand and K tile
+  static constexpr int CPT = 16 / NW;          // 1 KiB load instructions per wave and K tile for a 256-row operand stage
+  static constexpr int CPT_A = BM_ / 16 / NW;  // ... for the A stage of this tile height
 };
 constexpr int DL_BK = 32, DL_TILE_BYTES = 256 * DL_BK * 2;
 
@@ -869,9 +877,10 @@ __device__ __forceinline__ void wait_vm() {
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-template <bool TR, bool DUAL, int NW, bool MI16 = false>
+template <bool TR, bool DUAL, int NW, bool MI16 = false, int ROWS = 256>
 struct DlOperand {
-  static constexpr int CPT = DL<NW>::CPT, WN = DL<NW>::WN;
+  static_assert(ROWS == 256 || !TR, "a [k][row] stage is always 256 rows wide");
+  static constexpr int CPT = ROWS / 16 / NW, WN = DL<NW>::WN;
   unsigned voff[CPT];  // byte offset of this lane's 16-byte chunks from `base`
   const char* base;    // wave-uniform, advanced by `step` every K tile (DUAL: odd waves read the second matrix)
   int64_t step;
@@ -1057,12 +1066,13 @@ __device__ __forceinline__ void wait_tiles(int n) {
 }
 
 // PIX: the A operand is made from decoded frames (DlPixelOperand)
-template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, int NW, bool MI16 = false, bool PIX = false>
+template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, int NW, bool MI16 = false, bool PIX = false, int BM_ = 256>
 __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmParams p) {
   static_assert(!PIX || (!TA && !MI16 && !dl_prefetches(EPI, TA)), "frames as the A operand: [row][k] layout, 32x32x16 fragments, no early loads");
+  static_assert(BM_ == 256 || (!TA && !PIX && EPI != MVIT_EPI_SWIGLU_BWD), "half-height tiles: A in [row][k] layout, no per-256-row column sums");
   using T = bf16_t;
-  using D = DL<NW>;
-  constexpr int BM = D::BM, BN = D::BN, WM = D::WM, WN = D::WN, TILE = D::TILE_BYTES, SLICE = D::CPT * 1024;
+  using D = DL<NW, BM_>;
+  constexpr int BM = D::BM, BN = D::BN, WM = D::WM, WN = D::WN, TILE = D::TILE_BYTES, SLICE = D::CPT * 1024, SLICE_A = D::CPT_A * 1024;
   constexpr int MT = WM / 32, NT = WN / 32, WGN = BN / WN;
   constexpr bool DUAL = (EPI == MVIT_EPI_SWIGLU);
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -1077,7 +1087,8 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
   ra.init(wm * WM, 0);
   rb.init(wn * WN, NSTAGE * TILE);
   typedef __attribute__((address_space(3))) unsigned char lds_byte;
-  const unsigned lds0 = (unsigned)(__UINTPTR_TYPE__)(lds_byte*)smem_raw + wv * SLICE;
+  const unsigned lds0 = (unsigned)(__UINTPTR_TYPE__)(lds_byte*)smem_raw + wv * SLICE;      // this wave's slice of a B stage
+  const unsigned lds0a = (unsigned)(__UINTPTR_TYPE__)(lds_byte*)smem_raw + wv * SLICE_A;   // ... of an A stage
 
   // Persistent work-groups: the grid has at most one work-group per CU; work-group (xcd, slot) walks that XCD's
   // tile range with stride slots-per-XCD, the order a one-tile-per-work-group grid would be dispatched in.
@@ -1087,7 +1098,7 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
   constexpr bool PREFETCH = dl_prefetches(EPI, TA);
   constexpr int EARLY = PREFETCH ? (NSTAGE - 1 < 2 ? NSTAGE - 1 : 2) : NSTAGE - 1;  // K tiles requested by start_tile
   constexpr int STAGING_OFF = PREFETCH ? (NSTAGE + EARLY) * TILE : 0;
-  typename std::conditional<PIX, DlPixelOperand<NW>, DlOperand<TA, false, NW, MI16>>::type la;
+  typename std::conditional<PIX, DlPixelOperand<NW>, DlOperand<TA, false, NW, MI16, BM>>::type la;
   DlOperand<TB, DUAL, NW, MI16> lb;
   int T_ = 0, k_tail = 0;  // of the tile whose operands are being loaded
   [[maybe_unused]] int px_pending = -1;  // PIX: stage whose A bytes are in registers, requested by the previous issue()
@@ -1097,7 +1108,7 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
     if constexpr (PIX) {
       // the A bytes requested one call ago are converted and written now (their K tile is read two barriers from here),
       // then K tile t is requested: B straight into LDS, A into registers
-      if (px_pending >= 0) la.flush(smem_raw + px_pending * TILE + wv * SLICE, px_norm);
+      if (px_pending >= 0) la.flush(smem_raw + px_pending * TILE + wv * SLICE_A, px_norm);
       px_pending = -1;
       if (t >= T_) return;
       lb.issue(lds0 + (NSTAGE + s) * TILE);
@@ -1106,10 +1117,10 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
     } else {
       if (t >= T_) return;
       if (k_tail != 0 && t == T_ - 1) {
-        la.issue_tail(smem_raw + s * TILE + wv * SLICE, k_tail, wv);
+        la.issue_tail(smem_raw + s * TILE + wv * SLICE_A, k_tail, wv);
         lb.issue_tail(smem_raw + (NSTAGE + s) * TILE + wv * SLICE, k_tail, wv);
       } else {
-        la.issue(lds0 + s * TILE);
+        la.issue(lds0a + s * TILE);
         lb.issue(lds0 + (NSTAGE + s) * TILE);
       }
     }
@@ -1172,7 +1183,7 @@ __global__ __launch_bounds__(64 * NW, NW / 4) void gemm_dl_kernel(const GemmPara
       // tile t has landed once only the tiles issued after it are pending
       const int rem = T_ - 1 - t;
       constexpr int AHEAD = NSTAGE - 2;
-      wait_tiles<2 * D::CPT>(rem < 0 ? 0 : (rem < AHEAD ? rem : AHEAD));
+      wait_tiles<D::CPT_A + D::CPT>(rem < 0 ? 0 : (rem < AHEAD ? rem : AHEAD));
       __builtin_amdgcn_s_barrier();  // every wave's share of that tile is in LDS; stage (s-1) has been consumed
       // PIX: the conversion of the A bytes is vector work of about the length of a K tile's MFMAs.  The two waves of a
       // SIMD (w and w + NW/2) do it at opposite ends of the step, one before its MFMAs and one after, so that one
@@ -1327,16 +1338,28 @@ int launch(const GemmParams& p, hipStream_t stream) {
   return MVIT_OK;
 }
 
-template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, int NW, bool MI16 = false, bool PIX = false>
+// Compute units of the device (rounded down to a multiple of the 8 XCDs): persistent GEMM work-groups run one per unit.
+int device_cu_count(int dev) {
+  static int n_cu_on[MVIT_MAX_DEVICES] = {};
+  int& n_cu = n_cu_on[dev];
+  if (n_cu == 0) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+    n_cu = v / 8 * 8 > 0 ? v / 8 * 8 : 8;
+  }
+  return n_cu;
+}
+
+template <typename TO, bool TA, bool TB, int EPI, int NSTAGE, int NW, bool MI16 = false, bool PIX = false, int BM_ = 256>
 int launch_dl(const GemmParams& p, hipStream_t stream) {
-  using D = DL<NW>;
+  using D = DL<NW, BM_>;
   constexpr size_t operands = 2 * (size_t)NSTAGE * D::TILE_BYTES;
   constexpr size_t staging = (size_t)(D::BM / D::WM) * 32 * D::BN * sizeof(float);
   // with prefetching the staging area starts behind the B stages that the next tile's first two K tiles arrive in
   constexpr size_t staging_end = dl_prefetches(EPI, TA) ? (NSTAGE + (NSTAGE - 1 < 2 ? NSTAGE - 1 : 2)) * D::TILE_BYTES + staging : staging;
   constexpr size_t lds = staging_end > operands ? staging_end : operands;
   static_assert(lds <= 160 * 1024, "operand stages plus the epilogue staging area exceed the LDS of a CU");
-  auto kern = gemm_dl_kernel<TO, TA, TB, EPI, NSTAGE, NW, MI16, PIX>;
+  auto kern = gemm_dl_kernel<TO, TA, TB, EPI, NSTAGE, NW, MI16, PIX, BM_>;
   static bool attr_set_on[MVIT_MAX_DEVICES] = {};  // once per kernel and device
   const int dev = mvit_current_device("gemm");
   if (dev < 0) return MVIT_ERR_LAUNCH;
@@ -1348,13 +1371,7 @@ int launch_dl(const GemmParams& p, hipStream_t stream) {
   }
   if (p.split_k > 1 && EPI != MVIT_EPI_NONE) return mvit_set_error(MVIT_ERR_UNSUPPORTED, "gemm: split_k needs EPI_NONE");
   const int total = p.tiles_m * p.tiles_n * p.split_k;
-  static int n_cu_on[MVIT_MAX_DEVICES] = {};  // persistent work-groups: one per compute unit of the launching device
-  int& n_cu = n_cu_on[dev];
-  if (n_cu == 0) {
-    int v = 0;
-    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
-    n_cu = v / 8 * 8 > 0 ? v / 8 * 8 : 8;
-  }
+  const int n_cu = device_cu_count(dev);
   const int want = ((total + 7) / 8) * 8;
   const int grid = want < n_cu ? want : n_cu;
   hipLaunchKernelGGL(kern, grid, D::NTHREADS, lds, stream, p);
@@ -1561,6 +1578,23 @@ extern "C" int mvit_gemm(const mvit_gemm_args* a, mvit_stream_t stream) {
     }
   }
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  // Half-height tiles (128 x 256) for the two products that have few tile columns (N = hidden size): when the 256-row
+  // tiles would fill the last round of one-tile-per-unit work poorly and the 128-row tiles fill theirs better.  The
+  // result does not depend on the choice (same arithmetic per output element), so it may follow M.
+  if (a->dtype == MVIT_BF16 && a->out_dtype == MVIT_BF16 && var == 3 && !a->trans_a && p.split_k == 1 && getenv("MVIT_GEMM_NO_HALF_TILES") == nullptr &&
+      ((!a->trans_b && epi == MVIT_EPI_BIAS_RES) || (a->trans_b && epi == MVIT_EPI_NONE))) {
+    const int dev = mvit_current_device("gemm");
+    if (dev < 0) return MVIT_ERR_LAUNCH;
+    const double n_cu = device_cu_count(dev);
+    const int64_t tm_half = (a->M + 127) / 128;
+    const double r_full = (double)(tm * tn) / n_cu, r_half = (double)(tm_half * tn) / n_cu;
+    const double fill_full = r_full / ceil(r_full), fill_half = r_half / ceil(r_half);
+    if (fill_full < 0.75 && fill_half > fill_full + 0.1 && tm_half * tn < (1ll << 30)) {
+      p.tiles_m = (int)tm_half;
+      if (!a->trans_b) return launch_dl<bf16_t, false, false, MVIT_EPI_BIAS_RES, 4, 8, false, false, 128>(p, s);
+      return launch_dl<bf16_t, false, true, MVIT_EPI_NONE, 4, 8, true, false, 128>(p, s);
+    }
+  }
   if (a->dtype == MVIT_BF16) {
     if (a->out_dtype == MVIT_BF16) return dispatch_trans<bf16_t, bf16_t>(a->trans_a, a->trans_b, epi, var, p, s);
     return dispatch_trans<bf16_t, float>(a->trans_a, a->trans_b, epi, var, p, s);

@@ -344,6 +344,37 @@ def test_gemm_dgrad_layout(dtype, M, N, K):
     assert max_rel_err(out, a.double() @ w.double()[:, :N]) < TOL[dtype]
 
 
+@pytest.mark.parametrize("M", [4096, 16384, 1000, 130, 3408])
+@pytest.mark.parametrize("K", [1280, 3424])
+def test_gemm_half_height_tiles_give_the_same_bits_as_full_tiles(M, K, monkeypatch):
+    """Products with few tile columns (N = 1280) take 128-row tiles when 256-row tiles would leave most compute units
+    idle.  The choice follows M, so it must not change a single bit: same K order, same MFMA form, same epilogue."""
+    _announce(f"gemm half tiles M={M} K={K}")
+    ops = _ops()
+    from mi355_vit import _lib as E
+
+    N, dtype = 1280, torch.bfloat16
+    a, b = _rand((M, K), dtype, 0).to(DEV), _rand((N, K), dtype, 1, K**-0.5).to(DEV)
+    w = _rand((K, N), dtype, 4, K**-0.5).to(DEV)
+    bias, res = _rand((N,), dtype, 2).to(DEV), _rand((M, N), dtype, 3).to(DEV)
+
+    def run():
+        fwd = torch.full((M, N), 7.0, dtype=dtype, device=DEV)
+        dgrad = torch.full((M, N), 7.0, dtype=dtype, device=DEV)
+        ops.gemm(a, b, fwd, epilogue=E.EPI_BIAS_RES, bias=bias, residual=res)
+        ops.gemm(a, w, dgrad, trans_b=True)
+        torch.cuda.synchronize()
+        return fwd, dgrad
+
+    monkeypatch.setenv("MVIT_GEMM_NO_HALF_TILES", "1")
+    fwd_full, dgrad_full = run()
+    monkeypatch.delenv("MVIT_GEMM_NO_HALF_TILES")
+    fwd_half, dgrad_half = run()
+    assert torch.equal(fwd_half, fwd_full) and torch.equal(dgrad_half, dgrad_full)
+    assert max_rel_err(fwd_half, _gemm_ref(a.cpu(), b.cpu()) + bias.cpu().double() + res.cpu().double()) < TOL[dtype]
+    assert max_rel_err(dgrad_half, a.cpu().double() @ w.cpu().double()) < TOL[dtype]
+
+
 @pytest.mark.parametrize("dtype,odt", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32)])
 @pytest.mark.parametrize("S,No,Ni", [(1000, 1280, 1280), (515, 3840, 256), (70, 6848, 1280), (2052, 1280, 3420)])
 def test_gemm_wgrad_layout(dtype, odt, S, No, Ni):
