@@ -207,6 +207,54 @@ int mvit_attn_bwd(const void* q, const void* k, const void* v, const void* o, co
                   int64_t v_stride, int64_t o_stride, int64_t do_stride, int64_t dq_stride, int64_t dk_stride,
                   int64_t dv_stride, float scale, int dtype, mvit_stream_t stream);
 
+/* ---------------------------------------------------------------- one transformer block per call */
+
+/* Operands of one block (Qwen2_5_VLVisionBlock.forward, modeling:776-792, with _forward_standard :385-472 and the MLP
+ * :203-204) for mvit_block_fwd / mvit_block_bwd: the fixed launch sequence of the block behind one call each way, for
+ * hosts whose per-call cost would otherwise exceed the kernels' run time at small batches.  Every step is one of the
+ * entry points above on these operands, so the results are those of the same sequence issued call by call.
+ * All tensors are contiguous, of `dtype` unless a float* says otherwise; all pointers are device pointers.
+ *   weights  norm1, norm2 [C]; wqkv [3C, C], bqkv [3C] (q | k | v stacked); wproj [C, C], bproj [C];
+ *            wgu [2*Ipad, C], bgu [2*Ipad] (gate rows [0, I), up rows [Ipad, Ipad+I), padding rows zero);
+ *            wdown [C, Ipad] (padding columns zero), bdown [C]
+ *   geometry cu / seg_order / n_seg / max_seqlen as for mvit_attn_fwd; cos, sin fp32 [S, head_dim];
+ *            q_lead_scale = head_dim^-1/2 * log2 e applied to the queries in the rotary pass, attn_scale = 1 / log2 e
+ *   forward  x [S,C] in; written: n1 [S,C], rstd1 [S], qkv [S,3C], o [S,C] and lse [nheads,S] (read instead when
+ *            skip_attention != 0: the re-run of a checkpointed block that kept them), x1 [S,C], n2 [S,C], rstd2 [S],
+ *            gu [S,2*Ipad] (null: not saved, for a forward that will not be differentiated), h [S,Ipad],
+ *            x2 [S,C] (null: the down projection is skipped, for a re-run whose output nobody reads)
+ *   backward reads x and everything the forward wrote (gu required) plus dx2 [S,C]; writes dx [S,C], the parameter
+ *            gradients in `grad_dtype` laid out like the weights (g_wdown [C, I] without padding), and uses dgu
+ *            [S,2*Ipad], dn [S,C], dx1 [S,C], dqkv [S,3C] and `workspace` (mvit_block_bwd_workspace_bytes) as scratch.
+ *            split_k_*: K slices of the four weight-gradient GEMMs (>= 1).  side_stream (may be null): a second stream
+ *            of the caller's on which weight and bias gradients run beside the input-gradient chain; it then needs
+ *            five events of the caller's (hipEvent_t), and the call leaves the main stream waiting for the side one. */
+typedef struct mvit_block_args {
+  int dtype, grad_dtype;
+  int C, I, Ipad, nheads, head_dim;
+  int n_seg, max_seqlen, skip_attention;
+  int split_k_down, split_k_gate_up, split_k_proj, split_k_qkv;
+  float eps, q_lead_scale, attn_scale;
+  int64_t S;
+  const void *norm1, *norm2, *wqkv, *bqkv, *wproj, *bproj, *wgu, *bgu, *wdown, *bdown;
+  const int32_t *cu, *seg_order;
+  const float *cos, *sin;
+  const void* x;
+  void *n1, *qkv, *o, *x1, *n2, *gu, *h, *x2;
+  float *rstd1, *rstd2, *lse;
+  const void* dx2;
+  void *dx, *dgu, *dn, *dx1, *dqkv;
+  void *g_norm1, *g_norm2, *g_wqkv, *g_bqkv, *g_wproj, *g_bproj, *g_wgu, *g_bgu, *g_wdown, *g_bdown;
+  void* workspace;
+  int64_t workspace_bytes;
+  mvit_stream_t side_stream;
+  void* events[5];
+} mvit_block_args;
+
+int mvit_block_fwd(const mvit_block_args* args, mvit_stream_t stream);
+int64_t mvit_block_bwd_workspace_bytes(const mvit_block_args* args);
+int mvit_block_bwd(const mvit_block_args* args, mvit_stream_t stream);
+
 /* ---------------------------------------------------------------- vision -> text hand-off */
 
 /* Ranks the image placeholders of a token sequence: rank[t] = k (0-based) if input_ids[t] is the k-th entry equal

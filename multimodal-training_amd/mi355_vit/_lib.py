@@ -31,6 +31,24 @@ class GemmArgs(C.Structure):
     ]
 
 
+class BlockArgs(C.Structure):
+    """mvit_block_args: the operands of one transformer block for mvit_block_fwd / mvit_block_bwd."""
+
+    _fields_ = (
+        [(n, _i32) for n in ("dtype", "grad_dtype", "C", "I", "Ipad", "nheads", "head_dim", "n_seg", "max_seqlen", "skip_attention",
+                             "split_k_down", "split_k_gate_up", "split_k_proj", "split_k_qkv")]
+        + [(n, _f32) for n in ("eps", "q_lead_scale", "attn_scale")]
+        + [("S", _i64)]
+        + [(n, _vp) for n in ("norm1", "norm2", "wqkv", "bqkv", "wproj", "bproj", "wgu", "bgu", "wdown", "bdown",
+                              "cu", "seg_order", "cos", "sin", "x",
+                              "n1", "qkv", "o", "x1", "n2", "gu", "h", "x2", "rstd1", "rstd2", "lse",
+                              "dx2", "dx", "dgu", "dn", "dx1", "dqkv",
+                              "g_norm1", "g_norm2", "g_wqkv", "g_bqkv", "g_wproj", "g_bproj", "g_wgu", "g_bgu", "g_wdown", "g_bdown",
+                              "workspace")]
+        + [("workspace_bytes", _i64), ("side_stream", _vp), ("events", _vp * 5)]
+    )
+
+
 class AdamTensor(C.Structure):
     """mvit_adam_tensor: one row of the device-resident tensor table of the multi-tensor optimizer kernels."""
 
@@ -82,9 +100,11 @@ PROTOTYPES = {
     "mvit_resample_u8": [_vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _i32, _vp],
     "mvit_patch_embed_pack_weight": [_vp, _i32, _i64, _i64, _vp, _vp],
     "mvit_patch_embed_frames": [_vp, _i32, _i64, _vp, _i64, _vp, _i64, _i32, C.c_double] + [_f32] * 6 + [_vp],
+    "mvit_block_fwd": [C.POINTER(BlockArgs), _vp],
+    "mvit_block_bwd": [C.POINTER(BlockArgs), _vp],
     "mvit_attn_bwd": [_vp] * 10 + [_i64, _vp, _vp] + [_i32, _i32, _i64, _i32, _i32] + [_i64] * 8 + [_f32, _i32, _vp],
 }
-EXPORTS = sorted(list(PROTOTYPES) + ["mvit_version", "mvit_last_error", "mvit_attn_bwd_delta_elems"])
+EXPORTS = sorted(list(PROTOTYPES) + ["mvit_version", "mvit_last_error", "mvit_attn_bwd_delta_elems", "mvit_block_bwd_workspace_bytes"])
 HEADER_VERSION = 200  # MVIT_VERSION of include/mi355_vit.h these prototypes were written for
 
 _lib = None
@@ -110,6 +130,8 @@ def load() -> C.CDLL:
         lib.mvit_last_error.restype = C.c_char_p
         lib.mvit_attn_bwd_delta_elems.argtypes = [_i32, _i64, _i32, _i32, _i32]
         lib.mvit_attn_bwd_delta_elems.restype = _i64
+        lib.mvit_block_bwd_workspace_bytes.argtypes = [C.POINTER(BlockArgs)]
+        lib.mvit_block_bwd_workspace_bytes.restype = _i64
         if lib.mvit_version() != HEADER_VERSION:
             raise RuntimeError(f"{LIB_PATH} reports interface version {lib.mvit_version()}, these bindings are written for {HEADER_VERSION}: rebuild the library")
         _lib = lib

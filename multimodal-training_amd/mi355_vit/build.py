@@ -15,7 +15,7 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR.parent / "csrc"
 LIB_PATH = PKG_DIR / "libmi355vit.so"
-SOURCES = ["planners.cpp", "bandwidth.hip", "gemm.hip", "attention.hip", "optimizer.hip", "pixels.hip"]
+SOURCES = ["planners.cpp", "block.cpp", "bandwidth.hip", "gemm.hip", "attention.hip", "optimizer.hip", "pixels.hip"]
 
 # packed-fp32 instructions are switched off for every device translation unit
 HIPCC_FLAGS = [

@@ -10,6 +10,8 @@ Reference spans (python/models/qwen2_5_vl/modeling_qwen2_5_vl.py):
 
 from __future__ import annotations
 
+import ctypes
+import os
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Tuple
 
@@ -119,6 +121,108 @@ class AttnGeometry:
     order: Optional[torch.Tensor] = None  # device int32 permutation of the segments, longest first (ops.segment_order)
 
 
+# One C call per block and direction (mvit_block_fwd / mvit_block_bwd) instead of one per kernel: the same launches with
+# the same operands, issued from inside the library.  MVIT_BLOCK_CALLS=0 keeps the call-by-call sequence below, which is
+# also what runs while launches are being timed one by one (ops.set_trace) and for parameters of mixed gradient dtypes.
+BLOCK_CALLS = os.environ.get("MVIT_BLOCK_CALLS", "1") != "0"
+_join_events: dict = {}
+
+
+def _block_args(x: torch.Tensor, W: BlockWeights, geo: AttnGeometry, eps: float) -> "_lib.BlockArgs":
+    a = _lib.BlockArgs()
+    a.dtype = ops.dt(x)
+    a.S, a.C, a.I, a.Ipad, a.nheads, a.head_dim = x.shape[0], W.C, W.I, W.Ipad, geo.nheads, geo.head_dim
+    a.eps, a.q_lead_scale, a.attn_scale = eps, geo.head_dim**-0.5 * LOG2E, 1.0 / LOG2E
+    a.n_seg, a.max_seqlen = geo.cu.numel() - 1, geo.max_seqlen
+    a.norm1, a.norm2, a.wqkv, a.bqkv, a.wproj = W.norm1.data_ptr(), W.norm2.data_ptr(), W.wqkv.data_ptr(), W.bqkv.data_ptr(), W.wproj.data_ptr()
+    a.bproj, a.wgu, a.bgu, a.wdown, a.bdown = W.bproj.data_ptr(), W.wgu.data_ptr(), W.bgu.data_ptr(), W.wdown.data_ptr(), W.bdown.data_ptr()
+    a.cu, a.cos, a.sin = geo.cu.data_ptr(), geo.cos.data_ptr(), geo.sin.data_ptr()
+    a.seg_order = None if geo.order is None else geo.order.data_ptr()
+    a.x = x.data_ptr()
+    return a
+
+
+def _block_geometry_ok(x: torch.Tensor, W: BlockWeights, geo: AttnGeometry) -> bool:
+    """What the call-by-call wrappers check launch by launch, once for the block: operand layouts the C sequence assumes."""
+    S, hd = x.shape[0], geo.head_dim
+    return (x.is_cuda and x.is_contiguous() and x.shape[1] == W.C and geo.nheads * hd == W.C
+            and geo.cu.dtype == torch.int32 and geo.cu.is_contiguous() and geo.cu.device == x.device
+            and all(t.dtype == torch.float32 and tuple(t.shape) == (S, hd) and t.is_contiguous() for t in (geo.cos, geo.sin))
+            and (geo.order is None or (geo.order.dtype == torch.int32 and geo.order.is_contiguous() and geo.order.numel() == geo.cu.numel() - 1))
+            and all(t.is_contiguous() and t.dtype == x.dtype for t in (W.norm1, W.norm2, W.wqkv, W.bqkv, W.wproj, W.bproj, W.wgu, W.bgu, W.wdown, W.bdown)))
+
+
+def _block_forward_one_call(x, W, geo, eps, attn_out, for_backward, output):
+    S, C = x.shape
+    dev, T = x.device, x.dtype
+    f32 = torch.float32
+    n1, x1, n2 = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    rstd1, rstd2 = torch.empty(S, dtype=f32, device=dev), torch.empty(S, dtype=f32, device=dev)
+    qkv = torch.empty(S, 3 * C, dtype=T, device=dev)
+    if attn_out is None:
+        o, lse = torch.empty_like(x), torch.empty(geo.nheads, S, dtype=f32, device=dev)
+    else:
+        o, lse = attn_out
+    gu = torch.empty(S, 2 * W.Ipad, dtype=T, device=dev) if for_backward else None
+    h = torch.empty(S, W.Ipad, dtype=T, device=dev)
+    x2 = torch.empty_like(x) if output else None
+    a = _block_args(x, W, geo, eps)
+    a.skip_attention = int(attn_out is not None)
+    a.n1, a.qkv, a.o, a.x1, a.n2, a.h = n1.data_ptr(), qkv.data_ptr(), o.data_ptr(), x1.data_ptr(), n2.data_ptr(), h.data_ptr()
+    a.rstd1, a.rstd2, a.lse = rstd1.data_ptr(), rstd2.data_ptr(), lse.data_ptr()
+    a.gu, a.x2 = ops._p(gu), ops._p(x2)
+    _lib.check(_lib.load().mvit_block_fwd(ctypes.byref(a), ops._stream(x)), "mvit_block_fwd")
+    return x2, (rstd1, n1, qkv, o, lse, x1, rstd2, n2, gu, h)
+
+
+def _block_backward_one_call(dx2, x, saved, W, geo, gdt):
+    rstd1, n1, qkv, o, lse, x1, rstd2, n2, gu, h = saved
+    S, Cc = x.shape
+    I, Ipad = W.I, W.Ipad
+    dev, T = x.device, x.dtype
+    G = gdt["norm1.weight"]
+    e = lambda *shape, dtype=T: torch.empty(*shape, dtype=dtype, device=dev)  # noqa: E731
+    dx, dn, dx1 = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    dgu, dqkv = e(S, 2 * Ipad), e(S, 3 * Cc)
+    g_n1, g_n2, g_bp, g_bd = e(Cc, dtype=G), e(Cc, dtype=G), e(Cc, dtype=G), e(Cc, dtype=G)
+    g_wqkv, g_bqkv = e(3 * Cc, Cc, dtype=G), e(3 * Cc, dtype=G)
+    g_wp, g_wgu, g_bgu, g_wd = e(Cc, Cc, dtype=G), e(2 * Ipad, Cc, dtype=G), e(2 * Ipad, dtype=G), e(Cc, I, dtype=G)
+    a = _block_args(x, W, geo, 0.0)
+    a.grad_dtype = ops._DT[G]
+    a.n1, a.qkv, a.o, a.x1, a.n2, a.gu, a.h = n1.data_ptr(), qkv.data_ptr(), o.data_ptr(), x1.data_ptr(), n2.data_ptr(), gu.data_ptr(), h.data_ptr()
+    a.rstd1, a.rstd2, a.lse = rstd1.data_ptr(), rstd2.data_ptr(), lse.data_ptr()
+    a.dx2, a.dx, a.dgu, a.dn, a.dx1, a.dqkv = dx2.data_ptr(), dx.data_ptr(), dgu.data_ptr(), dn.data_ptr(), dx1.data_ptr(), dqkv.data_ptr()
+    a.g_norm1, a.g_norm2, a.g_wqkv, a.g_bqkv, a.g_wproj = g_n1.data_ptr(), g_n2.data_ptr(), g_wqkv.data_ptr(), g_bqkv.data_ptr(), g_wp.data_ptr()
+    a.g_bproj, a.g_wgu, a.g_bgu, a.g_wdown, a.g_bdown = g_bp.data_ptr(), g_wgu.data_ptr(), g_bgu.data_ptr(), g_wd.data_ptr(), g_bd.data_ptr()
+    sk = ops.wgrad_split_k
+    a.split_k_down, a.split_k_gate_up, a.split_k_proj, a.split_k_qkv = sk(Cc, I, S), sk(2 * Ipad, Cc, S), sk(Cc, Cc, S), sk(3 * Cc, Cc, S)
+    side = ops.side_stream(dev)
+    if side is not None:
+        key = dev.index if dev.index is not None else torch.cuda.current_device()
+        evs = _join_events.get(key)
+        if evs is None:
+            evs = [torch.cuda.Event() for _ in range(5)]
+            for ev in evs:
+                ev.record()  # an event object gets its handle with its first record
+            _join_events[key] = evs
+        a.side_stream = side.cuda_stream
+        for i, ev in enumerate(evs):
+            a.events[i] = ev.cuda_event
+    lib = _lib.load()
+    nbytes = lib.mvit_block_bwd_workspace_bytes(ctypes.byref(a))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), nbytes
+    _lib.check(lib.mvit_block_bwd(ctypes.byref(a), ops._stream(x)), "mvit_block_bwd")
+    grads = (
+        g_n1, g_n2,
+        g_wqkv[:Cc], g_bqkv[:Cc], g_wqkv[Cc : 2 * Cc], g_bqkv[Cc : 2 * Cc], g_wqkv[2 * Cc :], g_bqkv[2 * Cc :],
+        g_wp, g_bp,
+        g_wgu[:I], g_bgu[:I], g_wgu[Ipad : Ipad + I], g_bgu[Ipad : Ipad + I],
+        g_wd, g_bd,
+    )
+    return dx, grads
+
+
 def _block_forward(x: torch.Tensor, W: BlockWeights, geo: AttnGeometry, eps: float,
                    attn_out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, *,
                    for_backward: bool = True, output: bool = True) -> Tuple[Optional[torch.Tensor], tuple]:
@@ -129,6 +233,8 @@ def _block_forward(x: torch.Tensor, W: BlockWeights, geo: AttnGeometry, eps: flo
     pre-activations are not written (the first run of a checkpointed block).  ``output=False``: the block's output is
     not wanted, so the down projection is skipped (the re-run of a checkpointed block: the backward reads `h`, not
     `x2`)."""
+    if BLOCK_CALLS and ops._trace is None and _block_geometry_ok(x, W, geo):
+        return _block_forward_one_call(x, W, geo, eps, attn_out, for_backward, output)
     S, C = x.shape
     H, hd = geo.nheads, geo.head_dim
     n1, rstd1 = ops.rmsnorm_fwd(x, W.norm1.view(-1), eps)
@@ -167,6 +273,9 @@ def _block_backward(dx2: torch.Tensor, x: torch.Tensor, saved: tuple, W: BlockWe
     I, Ipad = W.I, W.Ipad
     dev = x.device
     dx2 = dx2.contiguous()
+    if (BLOCK_CALLS and ops._trace is None and len(set(gdt.values())) == 1 and gdt["norm1.weight"] in ops._DT and dx2.dtype == x.dtype
+            and _block_geometry_ok(x, W, geo)):
+        return _block_backward_one_call(dx2, x, saved, W, geo, gdt)
     main = torch.cuda.current_stream(dev)
     side = ops.side_stream(dev)
 

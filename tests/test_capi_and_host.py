@@ -67,6 +67,39 @@ def test_gemm_args_struct_matches_header_field_order():
     assert names == [f[0] for f in _lib.GemmArgs._fields_]
 
 
+def test_block_args_struct_matches_header_field_order_and_types():
+    import ctypes
+
+    from mi355_vit import _lib
+
+    header = (ROOT / "include" / "mi355_vit.h").read_text()
+    body = header[header.index("typedef struct mvit_block_args {") + len("typedef struct mvit_block_args {") : header.index("} mvit_block_args;")]
+    want = []
+    for stmt in body.split(";"):
+        stmt = " ".join(stmt.split())
+        if not stmt:
+            continue
+        m = re.match(r"(const )?(int64_t|int32_t|int|float|void|mvit_stream_t)\b(.*)", stmt)
+        assert m, stmt
+        base = m.group(2)
+        for name in m.group(3).split(","):
+            name = name.strip()
+            pointer = name.startswith("*") or base == "mvit_stream_t"
+            array = re.search(r"\[(\d+)\]", name)
+            name = re.sub(r"\[\d+\]", "", name.lstrip("* "))
+            if array:
+                ctype = ctypes.c_void_p * int(array.group(1))
+            elif pointer:
+                ctype = ctypes.c_void_p
+            else:
+                ctype = {"int": ctypes.c_int, "float": ctypes.c_float, "int64_t": ctypes.c_int64}[base]
+            want.append((name, ctype))
+    got = [(n, t) for n, t in _lib.BlockArgs._fields_]
+    assert [n for n, _ in got] == [n for n, _ in want]
+    for (n, t), (_, w) in zip(got, want):
+        assert ctypes.sizeof(t) == ctypes.sizeof(w) and (t is w or (t._type_ is w._type_ and t._length_ == w._length_) if hasattr(w, "_length_") else t is w), n
+
+
 def test_ops_refuse_cpu_tensors():
     from mi355_vit import ops
 

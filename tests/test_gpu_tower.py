@@ -151,6 +151,43 @@ def test_second_stream_overlap_gives_identical_gradients():
         assert torch.equal(res[0][1][k], res[1][1][k]), k
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("checkpoint", [False, True])
+def test_one_call_per_block_equals_the_call_by_call_sequence(dtype, checkpoint):
+    """mvit_block_fwd / mvit_block_bwd issue a block's launches from inside the library; the sequence issued call by call
+    (MVIT_BLOCK_CALLS=0, and what runs while launches are being timed) must give the same bits: output and every
+    gradient, plain and checkpointed, with the weight gradients on the second stream and in line."""
+    from mi355_vit import functional, ops
+
+    kw = dict(depth=3, hidden_size=512, intermediate_size=1200, num_heads=8, out_hidden_size=256, window_size=56, fullatt_block_indexes=[1])
+    g = torch.Generator().manual_seed(12)
+    grid = torch.tensor([[1, 32, 48], [1, 40, 28], [2, 16, 16]])
+    S = int((grid[:, 0] * grid[:, 1] * grid[:, 2]).sum())
+    pixels = torch.randn(S, 1176, generator=g)
+    gout = torch.randn(S // 4, 256, generator=g)
+    res = {}
+    old_calls, old_overlap = functional.BLOCK_CALLS, ops.OVERLAP_WGRAD
+    try:
+        for one_call in (True, False):
+            for overlap in (True, False):
+                functional.BLOCK_CALLS, ops.OVERLAP_WGRAD = one_call, overlap
+                model = _build(kw, 7, dtype)
+                if checkpoint:
+                    model.gradient_checkpointing_enable()
+                _run_gpu(model, pixels, grid, gout)
+                for p_ in model.parameters():
+                    p_.grad = None
+                res[(one_call, overlap)] = _run_gpu(model, pixels, grid, gout)  # second pass: buffers are recycled
+    finally:
+        functional.BLOCK_CALLS, ops.OVERLAP_WGRAD = old_calls, old_overlap
+    ref_out, ref_grads = res[(False, False)]
+    assert torch.isfinite(ref_out).all()
+    for key, (out, grads) in res.items():
+        assert torch.equal(out, ref_out), key
+        for k in ref_grads:
+            assert torch.equal(grads[k], ref_grads[k]), (key, k)
+
+
 def test_reference_smoke_shape():
     """The reference's own smoke case (tests/test_ragged_sp_smoke.py:27-98): output [192, 256]."""
     kw = dict(hidden_size=256, num_heads=8, depth=2, patch_size=14, in_channels=3, out_hidden_size=256, spatial_merge_size=2,
