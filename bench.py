@@ -454,7 +454,9 @@ def main() -> None:
 
     def step():
         model.zero_grad(set_to_none=True)
-        out = model(hidden_states=pixels, grid_thw=grid_dev)
+        # the grid goes in on the device and, as the trainer does, as the host copy it was made from (the model plans on
+        # the host; without the copy it reads the device tensor back and the host waits for the GPU once per step)
+        out = model(hidden_states=pixels, grid_thw=grid_dev, grid_thw_host=grid)
         out.backward(gout)
 
     def timed_steps(fn, warmup, steps, detail=None):
@@ -561,7 +563,7 @@ def main() -> None:
 
         def step2():
             model.zero_grad(set_to_none=True)
-            model(hidden_states=px, grid_thw=gd).backward(go)
+            model(hidden_states=px, grid_thw=gd, grid_thw_host=grid2).backward(go)
 
         torch.cuda.synchronize()
         torch.cuda.reset_peak_memory_stats()

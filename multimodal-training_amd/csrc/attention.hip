@@ -1245,22 +1245,9 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_x32(const AttnParams p) {
       lds_direct_16(lds_v0 + slot * (XS_TILE * 2) + wv * 1024, vv, V + (int64_t)ks * p.v_stride);
     }
   };
-  request_tile(0, 0);
-  request_tile(BK, 1);
-  request_tile(2 * BK, 2);
-  wait_vmcnt<0>();
-  __syncthreads();
-
   f32x16 o[QB][3];  // O^T: block mt, register i = head_dim 32*mt + 8*(i/4) + 4*hh + i%4 of query l%32; rows 80-95 = row sum of P
   float m_run[QB];
   f32x16 negm[QB];  // - m_run in every register: the accumulator input of the score product, so that scores arrive stabilised
-#pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    m_run[qb] = 0.f;
-    negm[qb] = splat16(0.f);
-#pragma unroll
-    for (int mt = 0; mt < 3; ++mt) o[qb][mt] = splat16(0.f);
-  }
 
   // V^T fragment (block mt of head_dim, contraction step ks): lane i of 16-lane group g4 supplies four consecutive
   // head-dim values of one key row; the transposing load hands lane j of the group head_dim 32*mt + 16*(g4 & 1) + j
@@ -1281,9 +1268,15 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_x32(const AttnParams p) {
 #pragma unroll
     for (int s = 0; s < ND; ++s) kf[s] = *reinterpret_cast<const bf16x8*>(lds_k[slot] + c32 * XS_PITCH + (((2 * s + hh) ^ xs16(c32)) << 3));
   };
-  fetch_k(0);
+  // One tile of 32 keys.  CHECK: the tile's row maxima are taken and the stabiliser follows them.  The first sweep over
+  // the keys does that for the first tile only and then leaves the stabiliser where it is: exp2 of a bf16 / fp32 value has
+  // 250 binary orders of range, so a later score may exceed the first tile's maximum by more than a hundred (base-2
+  // units) before anything overflows, and scores far below it vanish exactly as they would against the true maximum.
+  // A row whose sums did overflow is seen at the end (an infinity or NaN in its accumulators) and the work-group sweeps
+  // again with the maxima taken on every tile.
   int it = 0;
-  for (int k0 = 0; k0 < L; k0 += BK, ++it) {
+  auto tile_step = [&](int k0, auto check_tag) {
+    constexpr bool CHECK = decltype(check_tag)::value;
     const int b0 = it & (RING - 1), b1 = (it + 1) & (RING - 1), b3 = (it + 3) & (RING - 1);
     request_tile(k0 + 3 * BK, b3);
     const bf16_t* tv = lds_v[b0];
@@ -1344,8 +1337,7 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_x32(const AttnParams p) {
       sc[1] = mfma32x32(kf[1], qf[1][1], sc[1]);
       __builtin_amdgcn_sched_barrier(0);
       mask_tail(0);
-      const float mx0 = row_max(0);
-      rescale(0, mx0);
+      if constexpr (CHECK) rescale(0, row_max(0));
       __builtin_amdgcn_sched_barrier(0);
       sc[1] = mfma32x32(kf[2], qf[1][2], sc[1]);
       __builtin_amdgcn_sched_barrier(0);
@@ -1367,8 +1359,7 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_x32(const AttnParams p) {
       o[0][1] = mfma32x32(vf[1], p_operand(0, 0), o[0][1]);
       __builtin_amdgcn_sched_barrier(0);
       mask_tail(1);
-      const float mx1 = row_max(1);
-      rescale(1, mx1);
+      if constexpr (CHECK) rescale(1, row_max(1));
       __builtin_amdgcn_sched_barrier(0);
       o[0][2] = mfma32x32(vf[2], p_operand(0, 0), o[0][2]);
       __builtin_amdgcn_sched_barrier(0);
@@ -1395,6 +1386,37 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_x32(const AttnParams p) {
     if (k0 + 3 * BK < L) wait_vmcnt<2>();
     else wait_vmcnt<0>();
     __syncthreads();
+  };
+  auto sweep = [&](auto every_tile_tag) {
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      m_run[qb] = 0.f;
+      negm[qb] = splat16(0.f);
+#pragma unroll
+      for (int mt = 0; mt < 3; ++mt) o[qb][mt] = splat16(0.f);
+    }
+    request_tile(0, 0);
+    request_tile(BK, 1);
+    request_tile(2 * BK, 2);
+    wait_vmcnt<0>();
+    __syncthreads();
+    fetch_k(0);
+    it = 0;
+    tile_step(0, std::true_type{});
+    ++it;
+    for (int k0 = BK; k0 < L; k0 += BK, ++it) tile_step(k0, every_tile_tag);
+  };
+  sweep(std::false_type{});
+  {
+    // x * 0 is NaN for an infinity or a NaN and 0 otherwise: one chain of multiply-adds over a block's accumulators
+    float chk = 0.f;
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+      for (int mt = 0; mt < 3; ++mt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) chk = __builtin_fmaf(o[qb][mt][i], 0.f, chk);
+    if (__syncthreads_or(chk != chk)) sweep(std::true_type{});  // the ring is idle: every wave is past its last tile
   }
 
 #pragma unroll

@@ -282,8 +282,12 @@ class Qwen2_5_VisionTransformerPretrainedModel(nn.Module):
         idx, cu = ops.window_index(grid_thw, self.spatial_merge_size, self.window_size, self.patch_size)
         return idx.to(grid_thw.device), cu.tolist()
 
-    def _plan(self, grid_thw: torch.Tensor, device: torch.device) -> _TowerPlan:
-        grid = grid_thw.detach().to("cpu", torch.int64)
+    def _plan(self, grid_thw: torch.Tensor, device: torch.device, host: Optional[torch.Tensor] = None) -> _TowerPlan:
+        # the plan needs the grid on the host: a copy the caller still holds there (grids are born on the host, in the
+        # data pipeline) saves the device -> host read, which would make the host wait for all GPU work issued so far
+        grid = (host if host is not None else grid_thw).detach().to("cpu", torch.int64).reshape(-1, 3)
+        if host is not None and tuple(grid.shape) != tuple(grid_thw.reshape(-1, 3).shape):
+            raise ValueError(f"grid_thw_host {tuple(host.shape)} does not have the shape of grid_thw {tuple(grid_thw.shape)}")
         key = (tuple(grid.flatten().tolist()), str(device))
         plan = self._plans.get(key)
         if plan is None:
@@ -302,9 +306,11 @@ class Qwen2_5_VisionTransformerPretrainedModel(nn.Module):
 
     # ---- forward ---------------------------------------------------------------------------------
     def forward(self, hidden_states: Optional[torch.Tensor] = None, grid_thw: Optional[torch.Tensor] = None, *, frames=None,
-                **kwargs) -> torch.Tensor:
+                grid_thw_host: Optional[torch.Tensor] = None, **kwargs) -> torch.Tensor:
         """hidden_states: pixels view-able to [-1, in_channels*temporal_patch*patch*patch]; grid_thw [N,3] int64.
         Returns [S / merge^2, out_hidden_size] in the original (un-windowed) token order.
+        ``grid_thw_host`` (optional): the same values in a CPU tensor; a grid on the GPU is otherwise read back, which
+        makes the host wait for the GPU (the reference reads it back with ``.tolist()``, modeling:848, :876).
         ``frames`` (instead of ``hidden_states``; ``grid_thw`` then follows from their shapes): decoded, resized uint8
         frame stacks ``[frames, H, W, 3]`` on the GPU, one per image or video."""
         if self.sequence_parallel:
@@ -327,7 +333,7 @@ class Qwen2_5_VisionTransformerPretrainedModel(nn.Module):
             grid_thw = grid_of_frames
         elif grid_thw is None:
             raise ValueError("hidden_states needs grid_thw")
-        plan = self._plan(grid_thw, device)
+        plan = self._plan(grid_thw, device, grid_thw_host if frames is None else None)
         unit = self.spatial_merge_unit
 
         if frames is None:

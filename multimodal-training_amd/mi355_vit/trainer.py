@@ -362,6 +362,8 @@ class BaseVisionTrainer(Trainer):
             batch["image_grid_thw"] = grid_thw_of(batch["frames"])
         else:
             batch["pixel_values"] = batch["pixel_values"].to(device, non_blocking=True)
+        if not batch["image_grid_thw"].is_cuda:
+            batch["image_grid_thw_host"] = batch["image_grid_thw"]  # the model plans on the host: no read-back of the device copy
         batch["image_grid_thw"] = batch["image_grid_thw"].to(device, non_blocking=True)
         vision_outputs = self._model_forward(batch)
         forward_time_ms = 0.0
@@ -437,7 +439,7 @@ class BaseVisionTrainer(Trainer):
 
 class QwenVisionTrainer(BaseVisionTrainer):
     def _model_forward(self, batch):
-        pixel_values, grid = batch.get("pixel_values"), batch["image_grid_thw"]
+        pixel_values, grid, host = batch.get("pixel_values"), batch["image_grid_thw"], batch.get("image_grid_thw_host")
         with self._get_autocast_context():
             if pixel_values is None:  # uint8 frames: the model makes the patch rows itself
                 return self.model(frames=batch["frames"], grid_thw=grid).unsqueeze(0)
@@ -445,13 +447,15 @@ class QwenVisionTrainer(BaseVisionTrainer):
                 B = pixel_values.shape[0]
                 if grid.dim() == 1:
                     grid = grid.unsqueeze(0).expand(B, -1)
+                    host = None if host is None else host.unsqueeze(0).expand(B, -1)
                 elif grid.dim() == 2 and grid.shape[0] != B:
                     raise ValueError(f"image_grid_thw batch dimension {grid.shape[0]} doesn't match pixel_values batch dimension {B}")
-                out = self.model(hidden_states=pixel_values, grid_thw=grid)
+                out = self.model(hidden_states=pixel_values, grid_thw=grid, grid_thw_host=host)
                 return out.reshape(B, out.shape[0] // B, -1)
             if grid.dim() == 1:
                 grid = grid.unsqueeze(0)
-            return self.model(hidden_states=pixel_values, grid_thw=grid).unsqueeze(0)
+                host = None if host is None else host.unsqueeze(0)
+            return self.model(hidden_states=pixel_values, grid_thw=grid, grid_thw_host=host).unsqueeze(0)
 
 
 VisionTrainer = QwenVisionTrainer

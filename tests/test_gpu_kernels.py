@@ -143,6 +143,39 @@ def test_queries_scaled_in_the_rotary_pass_are_rounded_once():
     assert e_once < 2e-2 and e_once < 0.75 * e_twice and e_once < 1.5 * floor
 
 
+@pytest.mark.parametrize("late_key", [40, 1500, 2047])
+def test_attention_forward_scores_far_above_the_first_tiles(late_key):
+    """The long-segment forward sets its stabiliser from the first tile of keys and leaves it there; a later score that
+    exceeds it by more than the exponent range of exp2 overflows the row's sums, which the kernel sees at the end and
+    answers with a second sweep that follows the maxima tile by tile.  Here one late key scores about 190 base-2 units
+    above everything before it for every query: the result must still be the exact softmax (all weight on that key)."""
+    _announce(f"attention fwd: a score 190 binary orders above the first tile's maximum at key {late_key}")
+    ops = _ops()
+    S, H, d = 2048, 2, 80
+    g = torch.Generator().manual_seed(5)
+    u = torch.randn(H, d, generator=g)
+    u = u / u.norm(dim=1, keepdim=True)
+    q = (34.0 * u[None] + 0.1 * torch.randn(S, H, d, generator=g)).reshape(S, H * d).to(torch.bfloat16)
+    k = 0.1 * torch.randn(S, H, d, generator=g)
+    k[late_key] = 34.0 * u
+    k = k.reshape(S, H * d).to(torch.bfloat16)
+    v = torch.randn(S, H * d, generator=g).to(torch.bfloat16)
+    cu = torch.tensor([0, S], dtype=torch.int32, device=DEV)
+    o, lse = ops.attn_fwd(q.to(DEV), k.to(DEV), v.to(DEV), cu, S, H, d, d**-0.5)
+    heads = lambda t: t.double().reshape(S, H, d).transpose(0, 1)  # noqa: E731
+    scores = heads(q) @ heads(k).transpose(1, 2) * d**-0.5
+    assert float((scores[:, :, late_key] - scores[:, :, :32].amax(-1)).min()) * 1.4427 > 150.0  # the case is what it says
+    ref = (torch.softmax(scores, -1) @ heads(v)).transpose(0, 1).reshape(S, H * d)
+    assert torch.isfinite(o).all() and torch.isfinite(lse).all()
+    assert max_rel_err(o, ref) < TOL[torch.bfloat16]
+    assert max_rel_err(lse, torch.logsumexp(scores, -1)) < 5e-3  # the kernel rounds q * scale to bf16: 2^-9 of a score of 129
+    # the ordinary case next to it on the same launch shape: nothing overflows, one sweep
+    k2 = (0.1 * torch.randn(S, H * d, generator=g)).to(torch.bfloat16)
+    o2, _ = ops.attn_fwd(q.to(DEV), k2.to(DEV), v.to(DEV), cu, S, H, d, d**-0.5)
+    ref2 = (torch.softmax(heads(q) @ heads(k2).transpose(1, 2) * d**-0.5, -1) @ heads(v)).transpose(0, 1).reshape(S, H * d)
+    assert max_rel_err(o2, ref2) < TOL[torch.bfloat16]
+
+
 # ------------------------------------------------------------------------------------------ copies
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gather_rows_window_permutation_bit_exact(dtype):
