@@ -59,7 +59,7 @@ def _lr_lambda(kind: str, warmup: int, total: int):
         if kind == "linear":
             return max(0.0, 1.0 - prog)
         if kind == "cosine":
-            return max(0.0, 0.5 * (1.0 + math.cos(math.pi * min(1.0, prog))))
+            return max(0.0, 0.5 * (1.0 + math.cos(math.pi * prog)))  # not clamped past the last step: the library's half cosine rises again
         raise ValueError(f"unsupported lr_scheduler_type {kind!r}")
 
     return fn
@@ -184,7 +184,16 @@ class Trainer:
         ratio = self.config["warmup_ratio"]
         warmup = int(num_training_steps * ratio) if ratio > 0 else self.config["warmup_steps"]
         kind = self.config["lr_scheduler_type"]
-        self.scheduler = torch.optim.lr_scheduler.LambdaLR(self.optimizer, _lr_lambda(kind, warmup, num_training_steps))
+        if kind in ("linear", "cosine", "constant", "constant_with_warmup"):
+            self.scheduler = torch.optim.lr_scheduler.LambdaLR(self.optimizer, _lr_lambda(kind, warmup, num_training_steps))
+            return
+        # every other kind is the library's own schedule (the reference calls transformers.get_scheduler for all of
+        # them, python/ray/trainer.py:579-623); the four above are restated here so that they need no library
+        try:
+            from transformers import get_scheduler
+        except ImportError as exc:
+            raise ValueError(f"lr_scheduler_type {kind!r} needs transformers.get_scheduler, which is not importable here") from exc
+        self.scheduler = get_scheduler(name=kind, optimizer=self.optimizer, num_warmup_steps=warmup, num_training_steps=num_training_steps)
 
     # ---- helpers -----------------------------------------------------------------------------------
     def _get_torch_dtype(self, dtype_str: str = "bfloat16") -> torch.dtype:
@@ -319,8 +328,6 @@ class BaseVisionTrainer(Trainer):
     def set_receiver_info(self, receiver_gpu_ids, use_ipc: bool) -> None:
         self.receiver_gpu_ids = receiver_gpu_ids
         self.use_ipc = use_ipc
-        if use_ipc:
-            logger.warning("inter-process tensor hand-off is outside this build; embeddings are returned as tensors")
 
     # ---- steps ---------------------------------------------------------------------------------------
     def _model_forward(self, batch):
@@ -371,15 +378,28 @@ class BaseVisionTrainer(Trainer):
             torch.cuda.synchronize()
             forward_time_ms = (time.perf_counter() - t0) * 1000
         self._pending_outputs.append(vision_outputs)
-        return {"vision_embeddings": vision_outputs, "sample_index": sample_index, "iteration": iteration,
-                "forward_time_ms": forward_time_ms}
+        result = {"vision_embeddings": vision_outputs, "sample_index": sample_index, "iteration": iteration,
+                  "forward_time_ms": forward_time_ms}
+        if self.use_ipc and self.receiver_gpu_ids is not None:
+            # a receiver on the same GPU opens the embeddings in place (python/ray/vision.py:487-498): handles instead of
+            # the tensor, which stays alive in _pending_outputs until its backward
+            from .tensor_transfer import get_physical_gpu_id, prepare_tensor_for_transfer
+
+            request = prepare_tensor_for_transfer(vision_outputs.detach(), receiver_gpu_ids=self.receiver_gpu_ids,
+                                                  sender_gpu_id=get_physical_gpu_id(), use_ipc_if_same_gpu=True)
+            result["vision_embeddings"] = request.to_dict()
+        return result
 
     def _retrieve_gradient_tensor(self, vision_grad_ref):
+        """The gradient tensor out of what the text actor returned: a tensor, ``{"grad": ...}``, or a transfer request
+        whose handles are opened here (python/ray/vision.py:502-526; resolving a Ray object reference is the caller's)."""
         data = vision_grad_ref
         if isinstance(data, dict) and "grad" in data:
             data = data["grad"]
         if isinstance(data, dict) and "use_ipc" in data:
-            raise NotImplementedError("inter-process gradient hand-off is outside this build")
+            from .tensor_transfer import TensorTransferRequest, get_physical_gpu_id, receive_tensor
+
+            return receive_tensor(TensorTransferRequest.from_dict(data), get_physical_gpu_id())
         return data
 
     def _apply_vision_backward(self, vision_grad) -> None:

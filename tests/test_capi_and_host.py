@@ -260,3 +260,37 @@ def test_block_parameter_list_follows_the_declared_order():
     blk = model.blocks[0]
     blk.attn.proj.weight = torch.nn.Parameter(torch.zeros(64, 64))
     assert blk._block_params()[BLOCK_PARAM_ORDER.index("attn.proj.weight")] is blk.attn.proj.weight
+
+
+def test_transfer_request_round_trip_and_host_side_choices():
+    """python/ray/tensor_transfer.py:101-207 without a GPU: the dictionary form survives a round trip, and a tensor that
+    is not on a GPU (or a receiver elsewhere) travels as itself."""
+    from mi355_vit.tensor_transfer import TensorTransferRequest, get_physical_gpu_id, prepare_tensor_for_transfer, receive_tensor
+
+    t = torch.arange(6.0).reshape(2, 3)
+    req = prepare_tensor_for_transfer(t, ["gpu-a"], "gpu-a")
+    assert not req.use_ipc and req.tensor is t and req.ipc_handle is None  # host tensor: never by handle
+    back = TensorTransferRequest.from_dict(req.to_dict())
+    assert back.tensor is t and back.shape == t.shape and back.dtype == torch.float32 and back.sender_gpu_id == "gpu-a" and not back.use_ipc
+    assert receive_tensor(back, "gpu-b") is t
+    assert TensorTransferRequest.from_dict({"use_ipc": True, "dtype": "torch.bfloat16"}).dtype == torch.bfloat16
+    if not torch.cuda.is_available():
+        assert get_physical_gpu_id() == "cpu"
+
+
+@pytest.mark.parametrize("kind", ["linear", "cosine", "constant", "constant_with_warmup", "polynomial", "inverse_sqrt"])
+def test_schedules_equal_the_librarys(kind):
+    """The reference builds every schedule with transformers.get_scheduler (python/ray/trainer.py:579-623).  The four
+    kinds restated in the trainer must give the library's learning rates step for step; the others are the library's."""
+    transformers = pytest.importorskip("transformers")
+    tr = _host_trainer(lr_scheduler_type=kind, warmup_ratio=0.0, warmup_steps=3, learning_rate=2e-3)
+    tr._build_optimizer(list(tr.model.parameters()))
+    tr._build_scheduler(12)
+    ref_opt = torch.optim.Adam([torch.nn.Parameter(torch.zeros(1))], lr=2e-3)
+    ref = transformers.get_scheduler(name=kind, optimizer=ref_opt, num_warmup_steps=3, num_training_steps=12)
+    for _ in range(14):
+        assert tr.optimizer.param_groups[0]["lr"] == pytest.approx(ref_opt.param_groups[0]["lr"], rel=1e-12, abs=1e-18)
+        tr.optimizer.step()
+        tr.scheduler.step()
+        ref_opt.step()
+        ref.step()
