@@ -1061,18 +1061,30 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv_wide(const AttnParams p)
     BOps pb, db;
 #pragma unroll
     for (int s = 0; s < ND; ++s) {
+      // from the second step on the vector work is split between the two MFMAs: a wave issues in order, so whatever
+      // stands behind a second MFMA waits with it for the pipe, and only work placed between the two fills the first
+      // one's shadow.  (Step 0 keeps both MFMAs first: they separate group 0's last score MFMAs from the first read of
+      // their results, which the compiler does not guard.)
       if (s == 0) {
         mfma32x32_init(sc[1], qa[0], kf[1][0], nl);
         mfma32x32_init(dp[1], da[0], vf[1][0], nd);
-      } else {
+        words(0);
+        words(1);
+      } else if (s < 4) {
         mfma32x32_acc(sc[1], qa[s], kf[1][s]);
-        mfma32x32_acc(dp[1], da[s], vf[1][s]);
-      }
-      if (s < 4) {
+        __builtin_amdgcn_sched_barrier(0);
         words(2 * s);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma32x32_acc(dp[1], da[s], vf[1][s]);
+        __builtin_amdgcn_sched_barrier(0);
         words(2 * s + 1);
       } else {  // the lane swaps of group 0 under the last two score MFMAs
+        mfma32x32_acc(sc[1], qa[s], kf[1][s]);
+        __builtin_amdgcn_sched_barrier(0);
         pb = to_b_operands(pw);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma32x32_acc(dp[1], da[s], vf[1][s]);
+        __builtin_amdgcn_sched_barrier(0);
         db = to_b_operands(dw);
         asm volatile("s_nop 1");
       }
@@ -1585,17 +1597,23 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_wide(const AttnParams p) {
     BOps d0;
 #pragma unroll
     for (int s = 0; s < ND; ++s) {
+      // vector work between the two MFMAs from the second step on (see attn_bwd_dkdv_wide)
       if (s == 0) {
         mfma32x32_init(sc[1], ka[0], qf[1][0], nl[1]);
         mfma32x32_init(dp[1], va[0], dof[1][0], nd[1]);
-      } else {
+        word(0, 0);
+        word(0, 1);
+      } else if (s < 4) {
         mfma32x32_acc(sc[1], ka[s], qf[1][s]);
-        mfma32x32_acc(dp[1], va[s], dof[1][s]);
-      }
-      if (s < 4) {
+        __builtin_amdgcn_sched_barrier(0);
         word(0, 2 * s);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma32x32_acc(dp[1], va[s], dof[1][s]);
+        __builtin_amdgcn_sched_barrier(0);
         word(0, 2 * s + 1);
       } else {  // the lane swaps of block 0 under the last two score MFMAs
+        mfma32x32_acc(sc[1], ka[s], qf[1][s]);
+        mfma32x32_acc(dp[1], va[s], dof[1][s]);
         d0 = to_b_operands(dw[0]);
         asm volatile("s_nop 1");
       }
