@@ -294,3 +294,47 @@ def test_schedules_equal_the_librarys(kind):
         tr.scheduler.step()
         ref_opt.step()
         ref.step()
+
+
+def test_block_entry_points_refuse_malformed_arguments_before_any_launch():
+    """mvit_block_fwd / mvit_block_bwd check their struct on the host and return MVIT_ERR_ARG (-1) with a message; nothing
+    is launched, so made-up addresses are enough and no GPU is needed."""
+    import ctypes
+
+    from mi355_vit import _lib
+
+    lib = _lib.load()
+    assert lib.mvit_block_fwd(None, None) == -1 and b"null arguments" in lib.mvit_last_error()
+    a = _lib.BlockArgs()
+    assert lib.mvit_block_fwd(ctypes.byref(a), None) == -1 and b"bad sizes" in lib.mvit_last_error()
+    a.dtype, a.grad_dtype = _lib.BF16, _lib.BF16
+    a.S, a.C, a.I, a.Ipad, a.nheads, a.head_dim = 128, 256, 300, 304, 4, 64
+    assert lib.mvit_block_fwd(ctypes.byref(a), None) == -1 and b"null weight operand" in lib.mvit_last_error()
+    a.head_dim = 60  # heads x head_dim != C
+    assert lib.mvit_block_fwd(ctypes.byref(a), None) == -1 and b"bad sizes" in lib.mvit_last_error()
+    a.head_dim = 64
+    fake = 0x10000000
+    for name in ("norm1", "norm2", "wqkv", "bqkv", "wproj", "bproj", "wgu", "bgu", "wdown", "bdown"):
+        setattr(a, name, fake)
+    assert lib.mvit_block_fwd(ctypes.byref(a), None) == -1 and b"attention geometry missing" in lib.mvit_last_error()
+    a.cu, a.cos, a.sin, a.n_seg, a.max_seqlen = fake, fake, fake, 1, 128
+    assert lib.mvit_block_fwd(ctypes.byref(a), None) == -1 and b"null activation buffer" in lib.mvit_last_error()
+    for name in ("x", "n1", "rstd1", "qkv", "o", "lse", "x1", "n2", "rstd2", "h"):
+        setattr(a, name, fake)
+    # the backward wants more: saved factors, gradient buffers, slice counts, a workspace of the size it reports
+    assert lib.mvit_block_bwd(ctypes.byref(a), None) == -1 and b"null gradient buffer" in lib.mvit_last_error()
+    for name in ("gu", "dx2", "dx", "dgu", "dn", "dx1", "dqkv", "g_norm1", "g_norm2", "g_wqkv", "g_bqkv", "g_wproj", "g_bproj", "g_wgu", "g_bgu",
+                 "g_wdown", "g_bdown"):
+        setattr(a, name, fake)
+    assert lib.mvit_block_bwd(ctypes.byref(a), None) == -1 and b"split_k counts" in lib.mvit_last_error()
+    a.split_k_down = a.split_k_gate_up = a.split_k_proj = a.split_k_qkv = 2
+    need = lib.mvit_block_bwd_workspace_bytes(ctypes.byref(a))
+    assert need > 2 * 2 * 304 * 256 * 4  # at least the largest split-K workspace
+    a.workspace, a.workspace_bytes = fake, need - 1
+    assert lib.mvit_block_bwd(ctypes.byref(a), None) == -1 and b"workspace holds" in lib.mvit_last_error()
+    a.workspace_bytes = need
+    a.side_stream = fake  # a second stream without its events
+    assert lib.mvit_block_bwd(ctypes.byref(a), None) == -1 and b"five events" in lib.mvit_last_error()
+    a.S = 0  # an empty block is accepted and does nothing
+    a.side_stream = None
+    assert lib.mvit_block_fwd(ctypes.byref(a), None) == 0 and lib.mvit_block_bwd(ctypes.byref(a), None) == 0
