@@ -3,6 +3,7 @@ through inter-process memory and event handles, the second process hands the emb
 (python/ray/tensor_transfer.py:20-98, python/ray/vision.py:480-526).  The result must be bit-equal to the same step with
 both ends in one process."""
 
+import gc
 import os
 import subprocess
 import sys
@@ -39,8 +40,9 @@ while True:
     grad = (emb.float() * 0.5 + 1.0).to(emb.dtype)
     keep.append(grad)  # the sender of a tensor keeps it alive until the receiver is done
     back = prepare_tensor_for_transfer(grad, [request.sender_gpu_id], get_physical_gpu_id())
-    conn.send({"grad": back.to_dict(), "checksum": float(emb.double().sum()), "peer_gpu": get_physical_gpu_id()})
-    del emb
+    checksum = float(emb.double().sum())
+    del emb  # released before the answer leaves, so the sender finds nothing of its own still open here
+    conn.send({"grad": back.to_dict(), "checksum": checksum, "peer_gpu": get_physical_gpu_id()})
 conn.close()
 """
 
@@ -108,6 +110,11 @@ def test_embeddings_and_gradient_cross_a_process_boundary_without_a_copy():
                 torch.cuda.synchronize()
                 for n, p in tr.model.named_parameters():
                     assert torch.equal(p.grad, ref_grads[step][n]), (step, n)
+            # nothing of the peer's stays open here when the peer ends: a producer that exits first complains
+            del answer, res, handles
+            tr = None
+            gc.collect()
+            torch.cuda.ipc_collect()
             conn.send(None)
             conn.close()
             assert peer.wait(timeout=60) == 0
@@ -124,6 +131,8 @@ def test_a_receiver_on_another_gpu_is_refused_and_other_gpus_get_the_tensor_itse
     here = get_physical_gpu_id()
     plain = prepare_tensor_for_transfer(t, ["some-other-gpu"], here)
     assert not plain.use_ipc and plain.tensor is t and receive_tensor(plain, "some-other-gpu") is t
+    # (nobody opens this handle, so PyTorch's sender-side accounting reports an unreleased shared tensor when the test
+    # process ends; that line on stderr is about this request and nothing else)
     shared = prepare_tensor_for_transfer(t, [here], here)
     assert shared.use_ipc and shared.tensor is None and shared.shape == t.shape
     with pytest.raises(ValueError, match="only works for processes on the same physical GPU"):
